@@ -60,6 +60,10 @@ class CacheKind:
 
     paged = False
 
+    def is_paged(self, need) -> bool:
+        """Whether ``need`` lives in pages (the kind's ``paged`` unless a kind decides per need)."""
+        return self.paged
+
     def window(self, need) -> int | None:
         """Paged kinds: how many of the latest tokens a later query can still see (None: all)."""
         return None
@@ -153,6 +157,71 @@ class SlotState(CacheKind):
         binding.state.index_fill_(0, slots, 0)
 
 
+@dataclass
+class JointBinding:
+    """What the branches of a layer whose mixers run side by side are bound to, in the branches' order (None for a
+    branch that keeps nothing).  ``group`` is the paged branch's group."""
+
+    parts: list
+    group: int | None = None
+
+
+class JointMemory(CacheKind):
+    """The memory of mixers that run side by side (``parts.parallel.JointNeed``): each branch's need is sized,
+    allocated, shared and cleared by the kind it names itself.  At most one branch keeps pages."""
+
+    paged = True    # asked per need through ``is_paged``
+
+    def _paged(self, need):
+        found = [n for n in need.needs if n is not None and kind_of(n).is_paged(n)]
+        if len(found) > 1:
+            raise ValueError("mixers side by side: at most one of them may keep pages")
+        return found[0] if found else None
+
+    def is_paged(self, need):
+        return self._paged(need) is not None
+
+    def window(self, need):
+        n = self._paged(need)
+        return kind_of(n).window(n) if n is not None else None
+
+    def chunk(self, need):
+        n = self._paged(need)
+        return kind_of(n).chunk(n) if n is not None else None
+
+    def keeps_every_token(self, need):
+        return all(kind_of(n).keeps_every_token(n) for n in need.needs if n is not None)
+
+    def page_bytes(self, need, page_size, dtype):
+        return sum(kind_of(n).page_bytes(n, page_size, dtype) for n in need.needs if n is not None)
+
+    def request_bytes(self, need, dtype):
+        return sum(kind_of(n).request_bytes(n, dtype) for n in need.needs if n is not None)
+
+    def allocate(self, need, *, group, num_pages, page_size, num_slots, device, dtype):
+        parts = []
+        for n in need.needs:
+            if n is None:
+                parts.append(None)
+                continue
+            kind = kind_of(n)
+            paged = kind.is_paged(n)
+            parts.append(kind.allocate(n, group=group if paged else None, num_pages=num_pages if paged else 0,
+                                       page_size=page_size if paged else 0, num_slots=num_slots, device=device,
+                                       dtype=dtype))
+        binding = JointBinding(parts, group)
+        binding.kinds = [kind_of(n) if n is not None else None for n in need.needs]
+        return binding
+
+    def share(self, binding):
+        raise ValueError("mixers side by side keep memory that another run cannot read")
+
+    def reset(self, binding, slots):
+        for kind, part in zip(binding.kinds, binding.parts):
+            if part is not None:
+                kind.reset(part, slots)
+
+
 _KINDS: dict[type, CacheKind] = {}
 
 
@@ -180,3 +249,12 @@ def kind_of(need) -> CacheKind | None:
 register_cache_kind(KVCacheNeed, PagedKeysValues())
 register_cache_kind(LatentCacheNeed, PagedLatents())
 register_cache_kind(StateNeed, SlotState())
+
+
+def _register_joint() -> None:
+    from ..parts.parallel import JointNeed
+
+    register_cache_kind(JointNeed, JointMemory())
+
+
+_register_joint()

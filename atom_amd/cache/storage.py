@@ -43,7 +43,7 @@ def group_horizons(model) -> tuple[list[tuple], list[int | None]]:
     for run in model.order:
         need = model.blocks[run.layer].mixer.cache_need()
         kind = kind_of(need)
-        if kind is not None and kind.paged:
+        if kind is not None and kind.is_paged(need):
             window = (kind.window(need), kind.chunk(need))
             if window not in windows:
                 windows.append(window)
@@ -134,7 +134,7 @@ class CacheStorage:
         need = model.embedding.cache_need()
         if need is not None:
             kind = kind_of(need)
-            if kind.paged:
+            if kind.is_paged(need):
                 raise ValueError("an embedding's memory is per request, not paged")
             self.embedding_binding = kind.allocate(need, group=None, num_pages=0, page_size=0,
                                                    num_slots=num_state_slots, device=device, dtype=dtype)
@@ -145,7 +145,12 @@ class CacheStorage:
     @property
     def state_tensors(self) -> list[torch.Tensor]:
         """The per-request state tensors, in running order."""
-        return [b.state for _, b in self._owned if hasattr(b, "state")]
+        found = []
+        for _, b in self._owned:
+            for part in (getattr(b, "parts", None) or [b]):
+                if hasattr(part, "state"):
+                    found.append(part.state)
+        return found
 
     def reset_state(self, slots: list[int]) -> None:
         """Clears the per-request memory of slots whose requests start in this step."""

@@ -415,6 +415,118 @@ class RalitarConfig(ModelConfig):
         return out
 
 
+@dataclass(frozen=True)
+class LeduvikConfig(ModelConfig):
+    """``Leduvik``: token rows plus learned position rows; pre-norm layers listed one by one, each a mixer (a
+    selective state-space recurrence, windowed attention with unit-norm queries and keys, or attention and a
+    time-mixing recurrence side by side) and an optional dense feed-forward; a run of layers may be passed several
+    times, the embedding's output joining the stream again before every pass but the first.  config.json keys:
+    ``vocab``, ``width``, ``max_positions``, ``norm.eps``, ``logit_scale``, ``layers`` (``type``, ``mixer``,
+    ``mlp``), ``loop`` (``start``, ``stop``, ``times``)."""
+
+    layers: tuple = ()
+    norm_eps: float = 1e-6
+    logit_scale: float = 1.0
+    loop: tuple | None = None         # (start, stop, times)
+
+    model_type: ClassVar[str] = "leduvik"
+    MIXER_TYPES: ClassVar[tuple] = ("mamba2", "attention", "parallel")
+    MLP_KINDS: ClassVar[tuple] = ("dense",)
+
+    @classmethod
+    def from_dict(cls, raw: dict) -> "LeduvikConfig":
+        layers = _need(raw, "layers", list, "the model")
+        loop = raw.get("loop")
+        if loop is not None:
+            loop = tuple(_need(loop, k, int, "'loop'") for k in ("start", "stop", "times"))
+        cfg = cls(
+            architecture=raw.get("architecture") or (raw.get("architectures") or ["Leduvik"])[0],
+            vocab_size=_need(raw, "vocab", int, "the model"),
+            hidden_size=_need(raw, "width", int, "the model"),
+            num_hidden_layers=len(layers),
+            max_position_embeddings=_need(raw, "max_positions", int, "the model"),
+            tie_word_embeddings=False,
+            torch_dtype=str(raw.get("torch_dtype") or raw.get("dtype") or "bfloat16"),
+            bos_token_id=raw.get("bos_token_id"),
+            eos_token_id=raw.get("eos_token_id"),
+            layers=tuple(layers),
+            norm_eps=_need(raw.get("norm"), "eps", float, "'norm'"),
+            logit_scale=_take(raw, "logit_scale", float, 1.0),
+            loop=loop,
+        )
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if self.vocab_size <= 0 or self.hidden_size <= 0 or not self.layers:
+            raise ConfigError("vocab, width and the number of layers must be positive")
+        if self.max_position_embeddings <= 0:
+            raise ConfigError("max_positions must be positive")
+        if self.norm_eps <= 0:
+            raise ConfigError("norm.eps must be positive")
+
+        def positive(m, keys, where):
+            for key in keys:
+                if _need(m, key, int, where) <= 0:
+                    raise ConfigError(f"{where}: {key} must be positive")
+
+        def attention(m, where):
+            positive(m, ("heads", "kv_heads", "dim", "vdim"), where)
+            if m["heads"] % m["kv_heads"]:
+                raise ConfigError(f"{where}: heads must be a multiple of kv_heads")
+            _need(m, "scale", float, where)
+            mask = m.get("mask")
+            if mask is not None and _need(mask, "size", int, f"{where}'s mask") <= 0:
+                raise ConfigError(f"{where}: mask.size must be positive")
+            temp = m.get("q_temp")
+            if temp is not None:
+                _need(temp, "coef", float, f"{where}'s q_temp")
+                if _need(temp, "every", int, f"{where}'s q_temp") <= 0:
+                    raise ConfigError(f"{where}: q_temp.every must be positive")
+
+        for i, layer in enumerate(self.layers):
+            where = f"layer {i}"
+            kind = _need(layer, "type", str, where)
+            if kind not in self.MIXER_TYPES:
+                raise ConfigError(f"{where}: unknown type {kind!r}; known: {self.MIXER_TYPES}")
+            m = _need(layer, "mixer", dict, where)
+            mw = f"{where}'s mixer"
+            if kind == "mamba2":
+                positive(m, ("heads", "vdim", "state", "groups", "conv", "norm_groups"), mw)
+                if m["heads"] % m["groups"]:
+                    raise ConfigError(f"{where}: heads must be a multiple of groups")
+                if (m["heads"] * m["vdim"]) % m["norm_groups"]:
+                    raise ConfigError(f"{where}: heads * vdim must be a multiple of norm_groups")
+            elif kind == "attention":
+                attention(m, mw)
+            else:
+                attention(_need(m, "left", dict, mw), f"{mw}'s left")
+                positive(_need(m, "right", dict, mw), ("heads", "dim"), f"{mw}'s right")
+            mlp = layer.get("mlp")
+            if mlp is not None:
+                mk = _need(mlp, "kind", str, f"{where}'s mlp")
+                if mk not in self.MLP_KINDS:
+                    raise ConfigError(f"{where}: unknown mlp kind {mk!r}; known: {self.MLP_KINDS}")
+                positive(mlp, ("ff",), f"{where}'s mlp")
+        if self.loop is not None:
+            start, stop, times = self.loop
+            if not (0 <= start < stop <= len(self.layers)) or times < 1:
+                raise ConfigError(f"loop {self.loop} does not fit {len(self.layers)} layers")
+
+    def to_dict(self) -> dict:
+        out: dict[str, Any] = {
+            "architecture": self.architecture, "model_type": self.model_type, "vocab": self.vocab_size,
+            "width": self.hidden_size, "max_positions": self.max_position_embeddings, "norm": {"eps": self.norm_eps},
+            "logit_scale": self.logit_scale, "layers": [dict(layer) for layer in self.layers],
+        }
+        if self.loop is not None:
+            out["loop"] = dict(zip(("start", "stop", "times"), self.loop))
+        for key in ("bos_token_id", "eos_token_id"):
+            if getattr(self, key) is not None:
+                out[key] = getattr(self, key)
+        return out
+
+
 def read_config_json(folder: str) -> dict:
     path = os.path.join(folder, "config.json")
     if not os.path.isfile(path):

@@ -7,7 +7,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Callable
 
-from .model_config import ConfigError, LotoraxConfig, ModelConfig, Qwen3Config, RalitarConfig
+from .model_config import ConfigError, LeduvikConfig, LotoraxConfig, ModelConfig, Qwen3Config, RalitarConfig
 
 
 @dataclass(frozen=True)
@@ -79,3 +79,7 @@ def _ensure_builtin() -> None:
 
     if "Ralitar" not in _ARCHITECTURES:
         register_architecture("Ralitar", RalitarConfig, ralitar_spec)
+    from ..models.leduvik import leduvik_spec
+
+    if "Leduvik" not in _ARCHITECTURES:
+        register_architecture("Leduvik", LeduvikConfig, leduvik_spec)

@@ -1,0 +1,301 @@
+// Linear recurrences with a matrix state per head, and what stands around them.
+//
+// The state S of a head has K rows (key channels) and V columns (value channels), float32, and lives in the
+// request's state slot.  Per token, with a key k, a read vector r, a value v and a decay w (one per key channel, or
+// one per head):
+//
+//   read_before (a bonus u per key channel for the current token):
+//       o = (S + diag(u) k v^T)^T r;   S <- diag(w) S + k v^T
+//   read_after:
+//       S <- diag(w) S + k v^T;        o = S^T r
+//
+// v may first be multiplied by a step size per (token, head), and o may receive skip[h] * (the unscaled v).  The
+// columns of S never meet, so a column lives in registers, spread over LPC adjacent lanes of 16 rows each; r, k and w
+// of a run of tokens are staged in LDS by all lanes at once, the decay formed on the way (as given, or
+// exp(-exp(x + bias))).  A block is one wave: it owns 64 / LPC columns of one head of one request and walks the
+// request's tokens of this step in order, so a token's result depends on its own request only.
+//
+// Around it: token_shift (a token's input mixed with the previous token's, the previous token kept per request),
+// step_decay (softplus step sizes and the decays exp(-exp(A_log) dt) of a state-space layer), group_norm_gate (RMS
+// norm in equal parts of a row, a weight per entry, a SiLU gate before or after the norm).
+#include "common.h"
+
+constexpr int kScanRows = 16;    // rows of S a lane holds
+constexpr int kScanRun = 16;     // tokens staged at a time
+
+struct ScanArgs {
+  const float* r; long ldr; int r_div;       // head h reads r-head h / r_div, K entries each
+  const float* k; long ldk; int k_div;
+  const float* v; long ldv;                  // [T, H * V] at v
+  const float* w; long ldw; int w_per_channel;   // [T, H * K] or [T, H]
+  const float* w_bias; int w_mode;           // 0: w is the decay; 1: decay = exp(-exp(w + w_bias[h * K + i]))
+  const float* v_scale; long ldvs;           // [T, H] or null
+  const float* bonus;                        // [H, K]: read_before; null: read_after
+  const float* skip;                         // [H] or null
+  float* out; long ldo;                      // [T, H * V]
+  float* state; long slot_stride; long state_off;
+  const int* cu_seqlens; const int* slot_of_seq;
+  int H, K, V, lpc;
+};
+
+__global__ void __launch_bounds__(64) linear_scan_kernel(ScanArgs a) {
+  extern __shared__ float staged[];          // [kScanRun][3][KP]: r, k, w of a run's tokens
+  const int seq = blockIdx.x, h = blockIdx.y;
+  const int lpc = a.lpc, cols = kWave / lpc;
+  const int KP = lpc * kScanRows;
+  const int lane = threadIdx.x;
+  const int col = blockIdx.z * cols + lane / lpc;
+  const int part = lane % lpc;               // which 16 rows of the column
+  const int row0 = part * kScanRows;
+  const int t0 = a.cu_seqlens[seq], t1 = a.cu_seqlens[seq + 1];
+  const int slot = a.slot_of_seq[seq];
+  const bool live = col < a.V;
+  const int K = a.K, V = a.V;
+  if (slot < 0) {                            // a padding row: nothing to carry, its output is never read
+    for (int t = t0; t < t1; ++t)
+      if (live && part == 0) a.out[(size_t)t * a.ldo + (size_t)h * V + col] = 0.f;
+    return;
+  }
+  float* S_mem = a.state + (size_t)slot * a.slot_stride + a.state_off + (size_t)h * K * V;
+  float S[kScanRows];
+#pragma unroll
+  for (int i = 0; i < kScanRows; ++i) S[i] = (live && row0 + i < K) ? S_mem[(size_t)(row0 + i) * V + col] : 0.f;
+  float u[kScanRows];
+  const bool before = a.bonus != nullptr;
+#pragma unroll
+  for (int i = 0; i < kScanRows; ++i) u[i] = (before && row0 + i < K) ? a.bonus[(size_t)h * K + row0 + i] : 0.f;
+  const float skip = a.skip != nullptr ? a.skip[h] : 0.f;
+  const int rh = h / a.r_div, kh = h / a.k_div;
+
+  for (int base = t0; base < t1; base += kScanRun) {
+    const int n = min(kScanRun, t1 - base);
+    __syncthreads();
+    for (int e = lane; e < n * KP; e += kWave) {
+      const int j = e / KP, i = e - j * KP;
+      const size_t t = (size_t)(base + j);
+      float rv = 0.f, kv = 0.f, wv = 1.f;
+      if (i < K) {
+        rv = a.r[t * a.ldr + (size_t)rh * K + i];
+        kv = a.k[t * a.ldk + (size_t)kh * K + i];
+        wv = a.w_per_channel ? a.w[t * a.ldw + (size_t)h * K + i] : a.w[t * a.ldw + h];
+        if (a.w_mode == 1) wv = expf(-expf(wv + a.w_bias[(size_t)h * K + i]));
+      }
+      float* dst = staged + (size_t)j * 3 * KP;
+      dst[i] = rv;
+      dst[KP + i] = kv;
+      dst[2 * KP + i] = wv;
+    }
+    __syncthreads();
+    for (int j = 0; j < n; ++j) {
+      const size_t t = (size_t)(base + j);
+      const float* src = staged + (size_t)j * 3 * KP + row0;
+      const float v_raw = live ? a.v[t * a.ldv + (size_t)h * V + col] : 0.f;
+      const float v = a.v_scale != nullptr ? v_raw * a.v_scale[t * a.ldvs + h] : v_raw;
+      float acc = 0.f;
+      if (before) {
+#pragma unroll
+        for (int i = 0; i < kScanRows; ++i) {
+          const float kv = src[KP + i] * v;
+          acc += src[i] * (S[i] + u[i] * kv);
+          S[i] = src[2 * KP + i] * S[i] + kv;
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < kScanRows; ++i) {
+          S[i] = src[2 * KP + i] * S[i] + src[KP + i] * v;
+          acc += src[i] * S[i];
+        }
+      }
+      for (int off = lpc >> 1; off > 0; off >>= 1) acc += __shfl_xor(acc, off, kWave);
+      if (live && part == 0) a.out[t * a.ldo + (size_t)h * V + col] = acc + skip * v_raw;
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < kScanRows; ++i)
+      if (row0 + i < K) S_mem[(size_t)(row0 + i) * V + col] = S[i];
+  }
+}
+
+ATOM_EXPORT int atom_linear_scan(const float* r, long ldr, int r_div, const float* k, long ldk, int k_div, const float* v,
+                                 long ldv, const float* w, long ldw, int w_per_channel, const float* w_bias, int w_mode,
+                                 const float* v_scale, long ldvs, const float* bonus, const float* skip, float* out,
+                                 long ldo, float* state, long slot_stride, long state_off, const int* cu_seqlens,
+                                 const int* slot_of_seq, int num_seqs, int H, int K, int V, hipStream_t stream) {
+  if (H <= 0 || K <= 0 || V <= 0 || num_seqs < 0 || r_div <= 0 || k_div <= 0) return ATOM_BAD_SHAPE;
+  if (r == nullptr || k == nullptr || v == nullptr || w == nullptr || out == nullptr || state == nullptr) return ATOM_BAD_SHAPE;
+  if (cu_seqlens == nullptr || slot_of_seq == nullptr) return ATOM_BAD_SHAPE;
+  if (w_mode != 0 && w_mode != 1) return ATOM_UNSUPPORTED;
+  if (w_mode == 1 && (w_bias == nullptr || !w_per_channel)) return ATOM_BAD_SHAPE;
+  if (state_off < 0 || slot_stride < state_off + (long)H * K * V) return ATOM_BAD_SHAPE;
+  if (K > 16 * kScanRows) return ATOM_TOO_LARGE;
+  if (num_seqs == 0) return ATOM_OK;
+  int lpc = 1;
+  while (lpc * kScanRows < K) lpc <<= 1;
+  const int cols = kWave / lpc;
+  if (num_seqs > 0x7fffffff / 1 || H > 65535 || (V + cols - 1) / cols > 65535) return ATOM_TOO_LARGE;
+  ScanArgs a{r, ldr, r_div, k, ldk, k_div, v, ldv, w, ldw, w_per_channel, w_bias, w_mode, v_scale, ldvs, bonus, skip,
+             out, ldo, state, slot_stride, state_off, cu_seqlens, slot_of_seq, H, K, V, lpc};
+  const size_t smem = (size_t)kScanRun * 3 * lpc * kScanRows * sizeof(float);
+  hipLaunchKernelGGL(linear_scan_kernel, dim3(num_seqs, H, (V + cols - 1) / cols), dim3(kWave), smem, stream, a);
+  return launch_status();
+}
+
+// ------------------------------------------------------------------ a token's input mixed with the previous token's
+
+// mixes[s, t, :] = x[t] + (x[t - 1] - x[t]) * mu[s] for s < n; x[t - 1] of a request's first token of the step is
+// the row its state slot holds (zeros for a fresh request), and the step's last row of the request is left there.
+// The block of a request's first token reads the slot before it writes it, column by column.
+template <typename T>
+__global__ void __launch_bounds__(256)
+token_shift_kernel(const T* __restrict__ x, const float* __restrict__ mu, int n, T* __restrict__ mixes,
+                   float* __restrict__ state, long slot_stride, long state_off, const int* __restrict__ cu_seqlens,
+                   const int* __restrict__ slot_of_seq, const int* __restrict__ token_seq, int tokens, int width) {
+  const int t = blockIdx.x;
+  const int seq = token_seq[t];
+  const T* row = x + (size_t)t * width;
+  const bool padding = seq < 0;
+  const int first = padding ? t : cu_seqlens[seq];
+  const int slot = padding ? -1 : slot_of_seq[seq];
+  const bool heads = t == first;             // the request's first token of this step
+  const int last = padding ? t : cu_seqlens[seq + 1] - 1;
+  float* kept = slot >= 0 ? state + (size_t)slot * slot_stride + state_off : nullptr;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float cur = to_f32(row[i]);
+    float prev;
+    if (heads) {
+      prev = kept != nullptr ? kept[i] : 0.f;
+      if (kept != nullptr) kept[i] = to_f32(x[(size_t)last * width + i]);
+    } else {
+      prev = to_f32(x[(size_t)(t - 1) * width + i]);
+    }
+    const float d = prev - cur;
+    for (int s = 0; s < n; ++s)
+      mixes[((size_t)s * tokens + t) * width + i] = from_f32<T>(cur + d * mu[(size_t)s * width + i]);
+  }
+}
+
+ATOM_EXPORT int atom_token_shift(const void* x, int dtype, const float* mu, int n, void* mixes, float* state,
+                                 long slot_stride, long state_off, const int* cu_seqlens, const int* slot_of_seq,
+                                 const int* token_seq, int tokens, int width, hipStream_t stream) {
+  if (tokens < 0 || width <= 0 || n <= 0 || state_off < 0 || slot_stride < state_off + width) return ATOM_BAD_SHAPE;
+  if (x == nullptr || mu == nullptr || mixes == nullptr || state == nullptr) return ATOM_BAD_SHAPE;
+  if (cu_seqlens == nullptr || slot_of_seq == nullptr || token_seq == nullptr) return ATOM_BAD_SHAPE;
+  if (tokens == 0) return ATOM_OK;
+  ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((token_shift_kernel<T>), dim3(tokens), dim3(256), 0, stream, (const T*)x, mu,
+                                                 n, (T*)mixes, state, slot_stride, state_off, cu_seqlens, slot_of_seq,
+                                                 token_seq, tokens, width));
+  return launch_status();
+}
+
+// ------------------------------------------------------------------ step sizes and decays of a state-space layer
+
+// dt[t, h] = softplus(raw[t, h] + dt_bias[h]) (no clamp), decay[t, h] = exp(-exp(A_log[h]) dt[t, h]).
+__global__ void step_decay_kernel(const float* __restrict__ raw, long ld, const float* __restrict__ dt_bias,
+                                  const float* __restrict__ a_log, float* __restrict__ dt, float* __restrict__ decay,
+                                  int heads, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t t = idx / heads;
+  const int h = (int)(idx - t * heads);
+  const float z = raw[t * ld + h] + dt_bias[h];
+  const float step = z > 20.f ? z : log1pf(expf(z));
+  dt[idx] = step;
+  decay[idx] = expf(-expf(a_log[h]) * step);
+}
+
+ATOM_EXPORT int atom_step_decay(const float* raw, long ld, const float* dt_bias, const float* a_log, float* dt,
+                                float* decay, int tokens, int heads, hipStream_t stream) {
+  if (tokens < 0 || heads <= 0 || ld < heads) return ATOM_BAD_SHAPE;
+  if (raw == nullptr || dt_bias == nullptr || a_log == nullptr || dt == nullptr || decay == nullptr) return ATOM_BAD_SHAPE;
+  const size_t total = (size_t)tokens * heads;
+  if (total == 0) return ATOM_OK;
+  const size_t blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffffu) return ATOM_TOO_LARGE;
+  hipLaunchKernelGGL(step_decay_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, raw, ld, dt_bias, a_log, dt, decay,
+                     heads, total);
+  return launch_status();
+}
+
+// ------------------------------------------------------------------ RMS norm in equal parts of a row, with a gate
+
+// out[t, g, :] = y / rms(y) * weight * silu(gate)      (gate_first 0: the gate multiplies the normed row)
+// out[t, g, :] = z / rms(z) * weight, z = y * silu(gate) (gate_first 1: the gate comes before the norm)
+// for each of `groups` equal parts of a row of y (float32); gate: float32 [T, ldg], the row's gate values from
+// column 0 (null: no gate); weight: float32 [groups * gw] (null: ones).  A block a token; a part no wider than 256 is summed
+// by one wave, a wider one by the whole block.
+__device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+group_norm_gate_kernel(const float* __restrict__ y, long ldy, const float* __restrict__ gate, long ldg,
+                       const float* __restrict__ weight, T* __restrict__ out, int groups, int gw, float eps,
+                       int gate_first) {
+  __shared__ float scratch[16];
+  const size_t t = blockIdx.x;
+  const float* yr = y + t * ldy;
+  const float* gr = gate != nullptr ? gate + t * ldg : nullptr;
+  T* dst = out + t * (size_t)groups * gw;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave, waves = blockDim.x / kWave;
+  if (gw <= 256) {
+    for (int g = wave; g < groups; g += waves) {
+      const int base = g * gw;
+      float vals[4];
+      float ss = 0.f;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int i = lane + r * kWave;
+        float v = 0.f;
+        if (i < gw) {
+          v = yr[base + i];
+          if (gate_first && gr != nullptr) v *= silu_f(gr[base + i]);
+        }
+        vals[r] = v;
+        ss += v * v;
+      }
+      const float inv = 1.f / sqrtf(wave_sum(ss) / (float)gw + eps);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int i = lane + r * kWave;
+        if (i < gw) {
+          float v = vals[r] * inv;
+          if (weight != nullptr) v *= weight[base + i];
+          if (!gate_first && gr != nullptr) v *= silu_f(gr[base + i]);
+          dst[base + i] = from_f32<T>(v);
+        }
+      }
+    }
+    return;
+  }
+  for (int g = 0; g < groups; ++g) {
+    const int base = g * gw;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < gw; i += blockDim.x) {
+      float v = yr[base + i];
+      if (gate_first && gr != nullptr) v *= silu_f(gr[base + i]);
+      ss += v * v;
+    }
+    const float inv = 1.f / sqrtf(block_sum(ss, scratch) / (float)gw + eps);
+    for (int i = threadIdx.x; i < gw; i += blockDim.x) {
+      float v = yr[base + i];
+      const float s = gr != nullptr ? silu_f(gr[base + i]) : 1.f;
+      if (gate_first) v *= s;
+      v *= inv;
+      if (weight != nullptr) v *= weight[base + i];
+      if (!gate_first) v *= s;
+      dst[base + i] = from_f32<T>(v);
+    }
+  }
+}
+
+ATOM_EXPORT int atom_group_norm_gate(const float* y, long ldy, const float* gate, long ldg, const float* weight, void* out,
+                                     int out_dtype, int tokens, int groups, int gw, float eps, int gate_first,
+                                     hipStream_t stream) {
+  if (tokens < 0 || groups <= 0 || gw <= 0 || ldy < (long)groups * gw) return ATOM_BAD_SHAPE;
+  if (gate != nullptr && ldg < (long)groups * gw) return ATOM_BAD_SHAPE;
+  if (y == nullptr || out == nullptr) return ATOM_BAD_SHAPE;
+  if (tokens == 0) return ATOM_OK;
+  ATOM_DISPATCH_DTYPE(out_dtype, hipLaunchKernelGGL((group_norm_gate_kernel<T>), dim3(tokens), dim3(256), 0, stream, y, ldy,
+                                                     gate, ldg, weight, (T*)out, groups, gw, eps, gate_first));
+  return launch_status();
+}

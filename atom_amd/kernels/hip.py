@@ -195,7 +195,9 @@ class HipKernels:
                    "atom_experts_grouped", "atom_experts_grouped_tiles", "atom_experts_grouped_supports",
                    "atom_heads_gemm_mfma", "atom_heads_gemm_mfma_supports", "atom_rmsnorm_post", "atom_rmsnorm_rows",
                    "atom_cast_rows", "atom_token_gate", "atom_embedding_bigram", "atom_rglru_scan",
-                   "atom_keys_as_values_write", "atom_sigmoid_gate", "atom_bias_rows"):
+                   "atom_keys_as_values_write", "atom_sigmoid_gate", "atom_bias_rows", "atom_linear_scan", "atom_token_shift",
+                   "atom_step_decay", "atom_group_norm_gate", "atom_qkv_plain_write", "atom_narrow_heads",
+                   "atom_mean_of_norms", "atom_embedding_positions", "atom_unary_act", "atom_stream_add", "atom_scale_rows"):
             getattr(self.lib, fn).restype = ctypes.c_int
         self.allow_library_gemm = True
         # bfloat16 products of few rows run this library's own weight-streaming kernels: up to 64 rows, and
@@ -1076,7 +1078,7 @@ class HipKernels:
     # ------------------------------------------------------------------ the gated delta rule
 
     def conv_silu_state(self, x, channels: int, taps_weight, state, cu_seqlens_q, slot_of_seq, out,
-                        max_q_len: int | None = None, bias=None, activation: str = "silu"):
+                        max_q_len: int | None = None, bias=None, activation: str = "silu", x_offset: int = 0):
         """Short causal convolution per channel over each request's tokens (plus ``bias`` per channel when given),
         then SiLU (``activation`` "none": nothing).  ``x`` float32 [tokens, >=
         channels] (the first ``channels`` columns are convolved); ``taps_weight`` [channels, taps], last column the
@@ -1096,10 +1098,10 @@ class HipKernels:
             self._check("convolution bias", bias, torch.float32, (channels,))
         if activation not in ("silu", "none"):
             raise KernelError(f"conv_silu_state: unknown activation {activation!r}")
-        if ldx < channels or state.shape[1] < (taps - 1) * channels:
+        if x_offset < 0 or ldx < x_offset + channels or state.shape[1] < (taps - 1) * channels:
             raise KernelError("conv_silu_state: the input or the state is narrower than the channels need")
         self._done("conv_silu_state", self.lib.atom_conv_silu_state(
-            _ptr(x), ldx, _ptr(taps_weight), self._code(taps_weight), taps, channels, _ptr(state),
+            ctypes.c_void_p(x.data_ptr() + 4 * x_offset), ldx, _ptr(taps_weight), self._code(taps_weight), taps, channels, _ptr(state),
             ctypes.c_long(state.shape[1]), _ptr(cu_seqlens_q), _ptr(slot_of_seq), seqs,
             tokens if max_q_len is None else min(tokens, max_q_len), _ptr(out), _ptr(bias),
             0 if activation == "silu" else 1, self._stream()))
@@ -1152,6 +1154,210 @@ class HipKernels:
             self._code(out), tokens, heads, vdim, 0 if activation == "silu" else 1, self._stream()))
         return out
 
+    # ------------------------------------------------------------------ linear recurrences with a matrix state
+
+    @staticmethod
+    def _at(t: torch.Tensor, offset: int):
+        return ctypes.c_void_p(t.data_ptr() + t.element_size() * offset)
+
+    def linear_scan(self, r, r_off: int, r_heads: int, k, k_off: int, k_heads: int, v, v_off: int, w, w_off: int,
+                    state, state_off: int, cu_seqlens_q, slot_of_seq, out, heads: int, dim: int, vdim: int,
+                    per_channel: bool = True, w_bias=None, v_scale=None, bonus=None, skip=None):
+        """A linear recurrence with a state of ``dim`` x ``vdim`` per head over each request's tokens:
+        ``S <- diag(w) S + k v^T`` with the read-out ``o = (S_before + diag(bonus) k v^T)^T r`` where ``bonus``
+        [heads, dim] is given, else ``o = S_after^T r``.  All inputs float32 [tokens, *], read from a column offset:
+        ``r`` and ``k`` hold ``r_heads`` / ``k_heads`` heads of ``dim`` entries (head h reads head
+        ``h // (heads / r_heads)``), ``v`` ``heads`` x ``vdim``, ``w`` the decays, ``heads`` x ``dim`` with
+        ``per_channel`` and else one per head; with ``w_bias`` [heads, dim] the decay is ``exp(-exp(w + w_bias))``.
+        ``v_scale`` [tokens, heads] multiplies v on its way into the state; ``skip`` [heads] adds ``skip * v`` (v as
+        given) to the read-out.  The heads' matrices [heads, dim, vdim] start at ``state_off`` of a slot's row of
+        ``state``; requests with slot -1 are padding.  ``out`` float32 [tokens, heads * vdim]."""
+        tokens = out.shape[0]
+        seqs = slot_of_seq.numel()
+        if heads % r_heads or heads % k_heads:
+            raise KernelError("linear_scan: the heads are not a multiple of the r or k heads")
+        for name, t, off, wide in (("r", r, r_off, r_heads * dim), ("k", k, k_off, k_heads * dim),
+                                   ("v", v, v_off, heads * vdim), ("w", w, w_off, heads * (dim if per_channel else 1))):
+            self._check(f"scan {name}", t, torch.float32, (tokens, None))
+            if off < 0 or off + wide > t.shape[1]:
+                raise KernelError(f"linear_scan: {name} does not fit its tensor")
+        self._check("scan out", out, torch.float32, (tokens, heads * vdim))
+        self._check("state", state, torch.float32, (None, None))
+        self._check("cu_seqlens_q", cu_seqlens_q, torch.int32, (seqs + 1,))
+        self._check("slot_of_seq", slot_of_seq, torch.int32, (seqs,))
+        if w_bias is not None:
+            self._check("decay bias", w_bias, torch.float32, (heads * dim,))
+        if v_scale is not None:
+            self._check("step sizes", v_scale, torch.float32, (tokens, heads))
+        if bonus is not None:
+            self._check("bonus", bonus, torch.float32, (heads, dim))
+        if skip is not None:
+            self._check("skip", skip, torch.float32, (heads,))
+        L = ctypes.c_long
+        self._done("linear_scan", self.lib.atom_linear_scan(
+            self._at(r, r_off), L(r.shape[1]), heads // r_heads, self._at(k, k_off), L(k.shape[1]), heads // k_heads,
+            self._at(v, v_off), L(v.shape[1]), self._at(w, w_off), L(w.shape[1]), int(bool(per_channel)), _ptr(w_bias),
+            1 if w_bias is not None else 0, _ptr(v_scale), L(heads), _ptr(bonus), _ptr(skip), _ptr(out),
+            L(heads * vdim), _ptr(state), L(state.shape[1]), L(state_off), _ptr(cu_seqlens_q), _ptr(slot_of_seq), seqs,
+            heads, dim, vdim, self._stream()))
+        return out
+
+    def token_shift(self, x, mu, mixes, state, state_off: int, cu_seqlens_q, slot_of_seq, token_seq):
+        """``mixes[s, t] = x[t] + (x[t - 1] - x[t]) * mu[s]``; the row before a request's first token of the step is
+        what its state slot holds at ``state_off`` (float32, zeros for a fresh request), and the request's last row
+        of the step is left there."""
+        tokens, width = x.shape
+        n = mu.shape[0]
+        seqs = slot_of_seq.numel()
+        self._check("shift input", x, (torch.float32, torch.bfloat16))
+        self._check("shift weights", mu, torch.float32, (n, width))
+        self._check("shifted mixes", mixes, x.dtype, (n, tokens, width))
+        self._check("state", state, torch.float32, (None, None))
+        self._check("cu_seqlens_q", cu_seqlens_q, torch.int32, (seqs + 1,))
+        self._check("slot_of_seq", slot_of_seq, torch.int32, (seqs,))
+        self._check("token_seq", token_seq, torch.int32, (tokens,))
+        self._done("token_shift", self.lib.atom_token_shift(
+            _ptr(x), self._code(x), _ptr(mu), n, _ptr(mixes), _ptr(state), ctypes.c_long(state.shape[1]),
+            ctypes.c_long(state_off), _ptr(cu_seqlens_q), _ptr(slot_of_seq), _ptr(token_seq), tokens, width,
+            self._stream()))
+        return mixes
+
+    def step_decay(self, raw, raw_off: int, dt_bias, a_log, dt, decay):
+        """``dt = softplus(raw + dt_bias)``, ``decay = exp(-exp(a_log) dt)`` per (token, head); ``raw`` float32
+        [tokens, *] read from column ``raw_off``."""
+        tokens, heads = dt.shape
+        self._check("raw step sizes", raw, torch.float32, (tokens, None))
+        if raw_off < 0 or raw_off + heads > raw.shape[1]:
+            raise KernelError("step_decay: the raw step sizes do not fit their tensor")
+        self._check("dt_bias", dt_bias, torch.float32, (heads,))
+        self._check("A_log", a_log, torch.float32, (heads,))
+        self._check("step sizes", dt, torch.float32, (tokens, heads))
+        self._check("decays", decay, torch.float32, (tokens, heads))
+        self._done("step_decay", self.lib.atom_step_decay(
+            self._at(raw, raw_off), ctypes.c_long(raw.shape[1]), _ptr(dt_bias), _ptr(a_log), _ptr(dt), _ptr(decay),
+            tokens, heads, self._stream()))
+        return dt, decay
+
+    def group_norm_gate(self, y, groups: int, weight, eps: float, out, gate=None, gate_off: int = 0,
+                        gate_first: bool = False):
+        """RMS norm of each of ``groups`` equal parts of a row of ``y`` (float32), times ``weight`` (one per entry;
+        None: ones), with a SiLU gate from column ``gate_off`` of ``gate`` (float32) that multiplies the row before
+        the norm (``gate_first``) or after it."""
+        tokens, width = y.shape
+        if width % groups:
+            raise KernelError(f"group_norm_gate: {width} entries do not split into {groups} equal parts")
+        self._check("rows to norm", y, torch.float32)
+        if weight is not None:
+            self._check("norm weight", weight, torch.float32, (width,))
+        self._check("normed rows", out, (torch.float32, torch.bfloat16), (tokens, width))
+        gp, ldg = None, 0
+        if gate is not None:
+            self._check("gate", gate, torch.float32, (tokens, None))
+            if gate_off < 0 or gate_off + width > gate.shape[1]:
+                raise KernelError("group_norm_gate: the gate does not fit its tensor")
+            gp, ldg = self._at(gate, gate_off), gate.shape[1]
+        self._done("group_norm_gate", self.lib.atom_group_norm_gate(
+            _ptr(y), ctypes.c_long(width), gp, ctypes.c_long(ldg), _ptr(weight), _ptr(out), self._code(out), tokens,
+            groups, width // groups, ctypes.c_float(eps), int(bool(gate_first)), self._stream()))
+        return out
+
+    # ------------------------------------------------------------------ attention without rotation
+
+    def qkv_plain_write(self, proj, q_out, k_cache, v_cache, positions, slots, num_heads: int, num_kv_heads: int,
+                        head_dim: int, value_dim: int, page_size: int, unit_norm: bool, eps: float,
+                        temperature: tuple | None = None, write_kv: bool = True):
+        """From the float32 product ``proj`` [tokens, q | k | v]: q (with ``unit_norm`` divided by each head's root
+        mean square, as k is; times the token's temperature ``1 + coef ln(floor((p + 1) / every) + 1)`` for
+        ``temperature`` = (coef, every)) to ``q_out`` [tokens, heads, padded], k and v to the pages, whose head
+        size ``padded`` >= max(head_dim, value_dim) is ``q_out``'s; what lies beyond a head's own entries is zero."""
+        tokens = proj.shape[0]
+        dp = q_out.shape[2]
+        dt = q_out.dtype
+        self._check("q|k|v", proj, torch.float32, (tokens, None))
+        if proj.shape[1] < (num_heads + num_kv_heads) * head_dim + num_kv_heads * value_dim:
+            raise KernelError("qkv_plain_write: the product is narrower than its heads")
+        self._check("q out", q_out, (torch.float32, torch.bfloat16), (tokens, num_heads, dp))
+        if dp < head_dim or dp < value_dim:
+            raise KernelError("qkv_plain_write: the padded head size is smaller than a head")
+        if write_kv:
+            self._check("key pages", k_cache, dt, (None, num_kv_heads, page_size, dp))
+            self._check("value pages", v_cache, dt, (k_cache.shape[0], num_kv_heads, dp, page_size))
+            self._check("slot mapping", slots, torch.int32, (tokens,))
+        coef, every = (float(temperature[0]), int(temperature[1])) if temperature else (0.0, 1)
+        if coef != 0.0:
+            if every <= 0:
+                raise KernelError("qkv_plain_write: the temperature's step must be positive")
+            self._check("positions", positions, torch.int32, (tokens,))
+        self._done("qkv_plain_write", self.lib.atom_qkv_plain_write(
+            _ptr(proj), ctypes.c_long(proj.shape[1]), _ptr(q_out), _ptr(k_cache) if write_kv else None,
+            _ptr(v_cache) if write_kv else None, self._code(q_out), _ptr(positions) if coef != 0.0 else None,
+            _ptr(slots) if write_kv else None, tokens, num_heads, num_kv_heads, head_dim, value_dim, dp, page_size,
+            int(bool(unit_norm)), ctypes.c_float(eps), ctypes.c_float(coef), every, self._stream()))
+        return q_out
+
+    def narrow_heads(self, x, value_dim: int):
+        """The first ``value_dim`` entries of every head of ``x`` [tokens, heads, padded], as [tokens, heads *
+        value_dim]."""
+        tokens, heads, dp = x.shape
+        self._check("padded heads", x, (torch.float32, torch.bfloat16))
+        if value_dim == dp:
+            return x.view(tokens, heads * dp)
+        out = torch.empty((tokens, heads * value_dim), dtype=x.dtype, device=x.device)
+        self._done("narrow_heads", self.lib.atom_narrow_heads(_ptr(x), _ptr(out), self._code(x),
+                                                              ctypes.c_long(tokens * heads), dp, value_dim, self._stream()))
+        return out
+
+    def mean_of_norms(self, xs, weights, eps: float, out):
+        """``out = mean_b(xs[b] / rms(xs[b]) * weights[b])`` over up to four inputs of ``out``'s shape and type."""
+        n = len(xs)
+        if not 1 <= n <= 4 or len(weights) != n:
+            raise KernelError("mean_of_norms: one to four inputs, a weight each")
+        tokens, width = out.shape
+        self._check("mean of norms", out, (torch.float32, torch.bfloat16))
+        xs = [self.materialize(x) for x in xs]
+        for x, w in zip(xs, weights):
+            self._check("normed input", x, out.dtype, (tokens, width))
+            self._check("norm weight", w, torch.float32, (width,))
+        xp = (ctypes.c_void_p * n)(*[x.data_ptr() for x in xs])
+        wp = (ctypes.c_void_p * n)(*[w.data_ptr() for w in weights])
+        self._done("mean_of_norms", self.lib.atom_mean_of_norms(xp, wp, n, _ptr(out), self._code(out), tokens, width,
+                                                                ctypes.c_float(eps), self._stream()))
+        return out
+
+    def embedding_positions(self, table, rows, ids, positions, out):
+        """``out = table[ids] + rows[positions]`` in float32."""
+        vocab, hidden = table.shape
+        tokens = ids.numel()
+        self._check("embedding table", table, (torch.float32, torch.bfloat16))
+        self._check("position rows", rows, table.dtype, (None, hidden))
+        self._check("token ids", ids, torch.int32, (tokens,))
+        self._check("positions", positions, torch.int32, (tokens,))
+        self._check("embedding out", out, torch.float32, (tokens, hidden))
+        self._done("embedding_positions", self.lib.atom_embedding_positions(
+            _ptr(table), _ptr(rows), self._code(table), _ptr(ids), _ptr(positions), _ptr(out), tokens, hidden, vocab,
+            rows.shape[0], self._stream()))
+        return out
+
+    def scale_rows(self, x, scale: float):
+        """``x *= scale`` in place for a float32 ``x``."""
+        self._check("rows to scale", x, torch.float32)
+        self._done("scale_rows", self.lib.atom_scale_rows(_ptr(x), ctypes.c_long(x.numel()), ctypes.c_float(scale),
+                                                          self._stream()))
+        return x
+
+    _UNARY = {"silu": 0, "relu": 1, "gelu_tanh": 2, "relu_squared": 3, "tanh": 4}
+
+    def unary_act(self, x, out, activation: str):
+        """``out = act(x)`` entry by entry."""
+        x = self.materialize(x)
+        if activation not in self._UNARY:
+            raise KernelError(f"unary_act: unknown activation {activation!r}; known: {sorted(self._UNARY)}")
+        self._check("activation input", x, (torch.float32, torch.bfloat16))
+        self._check("activation out", out, x.dtype, tuple(x.shape))
+        self._done("unary_act", self.lib.atom_unary_act(_ptr(x), _ptr(out), self._code(x), ctypes.c_long(x.numel()),
+                                                        self._UNARY[activation], self._stream()))
+        return out
+
     # ------------------------------------------------------------------ a float32 stream with normed summands
 
     def rmsnorm_post(self, x, weight, eps: float, stream, out=None):
@@ -1170,16 +1376,28 @@ class HipKernels:
         return out
 
     def rmsnorm_rows(self, x, weight, eps: float, rows, out):
-        """``out[r] = norm(x[rows[r]]) * weight`` for float32 ``x``, written in ``out``'s type."""
+        """``out[r] = norm(x[rows[r]]) * weight`` for float32 ``x``, written in ``out``'s type (``rows`` None: every
+        row in turn)."""
         n, width = x.shape
         self._check("norm input", x, torch.float32, (n, width))
         self._check("norm weight", weight, torch.float32, (width,))
-        self._check("norm rows", rows, torch.int32, (None,))
-        self._check("norm out", out, (torch.float32, torch.bfloat16), (rows.numel(), width))
+        if rows is not None:
+            self._check("norm rows", rows, torch.int32, (None,))
+        n_out = rows.numel() if rows is not None else n
+        self._check("norm out", out, (torch.float32, torch.bfloat16), (n_out, width))
         self._done("rmsnorm_rows", self.lib.atom_rmsnorm_rows(
-            _ptr(x), _ptr(weight), ctypes.c_float(eps), _ptr(rows), n, _ptr(out), self._code(out), rows.numel(), width,
+            _ptr(x), _ptr(weight), ctypes.c_float(eps), _ptr(rows), n, _ptr(out), self._code(out), n_out, width,
             self._stream()))
         return out
+
+    def stream_add(self, stream, x, init: bool = False):
+        """``stream += x`` (``init``: ``stream = x``) for a float32 ``stream`` and an ``x`` of any type."""
+        x = self.materialize(x)
+        self._check("stream", stream, torch.float32)
+        self._check("summand", x, (torch.float32, torch.bfloat16), tuple(stream.shape))
+        self._done("stream_add", self.lib.atom_stream_add(_ptr(stream), _ptr(x), self._code(x),
+                                                          ctypes.c_long(stream.numel()), int(bool(init)), self._stream()))
+        return stream
 
     def cast_rows(self, x, dtype):
         """Float32 rows in another type."""

@@ -4,19 +4,23 @@ from .base import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, JOINS, MIXERS, NORM
                    FeedForward, Head, Join, KVCacheNeed, LatentCacheNeed, Mixer, Norm, ParamSpec, Part, PartChoice,
                    PositionEncoding, Registry, Source, StateNeed)
 from . import (attention, block, delta, embedding, experts, join, kv_attention, latent_attention, mlp, norm,  # noqa: F401
-               rglru, rope, token_side)
+               parallel, plain_attention, rglru, rope, state_space, time_mix, token_side)
 from .attention import GroupedQueryAttention
 from .block import PostNormBlock, PreNormBlock, SandwichBlock
 from .delta import GatedDeltaRule
-from .embedding import BigramEmbedding, LMHead, ScaledEmbedding, TokenEmbedding
+from .embedding import BigramEmbedding, LMHead, PositionedEmbedding, ScaledEmbedding, TokenEmbedding
 from .experts import RoutedExperts
-from .join import ConcatProjection
+from .join import AddFirst, ConcatProjection
 from .kv_attention import KeyValueAttention
 from .latent_attention import LatentAttention
-from .mlp import GatedMLP
+from .mlp import DenseMLP, GatedMLP
 from .norm import LayerNorm, RMSNorm
+from .parallel import JointNeed, ParallelMixer
+from .plain_attention import PlainAttention
 from .rglru import RealGatedRecurrence
 from .rope import BandedRotary, RotaryEncoding, ScaledRotary
+from .state_space import StateSpaceMixer
+from .time_mix import TimeMixRecurrence
 from .token_side import TokenSide
 
 __all__ = [
@@ -26,5 +30,6 @@ __all__ = [
     "GroupedQueryAttention", "PreNormBlock", "LMHead", "TokenEmbedding", "GatedMLP", "RMSNorm", "RotaryEncoding",
     "SandwichBlock", "GatedDeltaRule", "ScaledEmbedding", "RoutedExperts", "ConcatProjection", "LatentAttention",
     "LayerNorm", "ScaledRotary", "PostNormBlock", "BigramEmbedding", "KeyValueAttention", "RealGatedRecurrence",
-    "BandedRotary", "TokenSide",
+    "BandedRotary", "TokenSide", "AddFirst", "DenseMLP", "JointNeed", "ParallelMixer", "PlainAttention",
+    "PositionedEmbedding", "StateSpaceMixer", "TimeMixRecurrence",
 ]

@@ -10,7 +10,7 @@ from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block, PartChoice
 
 
 class PreNormBlock(Block):
-    def __init__(self, mixer: PartChoice, feed_forward: PartChoice, norm: PartChoice, prefix: str = "",
+    def __init__(self, mixer: PartChoice, feed_forward: PartChoice | None, norm: PartChoice, prefix: str = "",
                  names: dict[str, str] | None = None):
         super().__init__(prefix)
         n = {"mixer_norm": "input_layernorm", "mixer": "self_attn", "ffn_norm": "post_attention_layernorm",
@@ -18,15 +18,16 @@ class PreNormBlock(Block):
         sub = lambda name: f"{prefix}.{n[name]}" if prefix else n[name]  # noqa: E731
         self.mixer_norm = norm.build(NORMS, prefix=sub("mixer_norm"))
         self._mixer = mixer.build(MIXERS, prefix=sub("mixer"))
-        self.ffn_norm = norm.build(NORMS, prefix=sub("ffn_norm"))
-        self.ffn = feed_forward.build(FEED_FORWARDS, prefix=sub("ffn"))
+        # ``feed_forward`` None: the layer is its mixer alone, and hands on the mixer's output
+        self.ffn = feed_forward.build(FEED_FORWARDS, prefix=sub("ffn")) if feed_forward is not None else None
+        self.ffn_norm = norm.build(NORMS, prefix=sub("ffn_norm")) if self.ffn is not None else None
 
     @property
     def mixer(self):
         return self._mixer
 
     def children(self):
-        return [self.mixer_norm, self._mixer, self.ffn_norm, self.ffn]
+        return [self.mixer_norm, self._mixer] + ([self.ffn_norm, self.ffn] if self.ffn is not None else [])
 
     def forward(self, ctx, hidden, residual, cache):
         if not self.mixer_norm.accepts_deferred:
@@ -35,6 +36,8 @@ class PreNormBlock(Block):
         if not self._mixer.accepts_deferred:
             hidden = ctx.ops.materialize(hidden)
         hidden = self._mixer.forward(ctx, hidden, cache)
+        if self.ffn is None:
+            return hidden, residual
         if not self.ffn_norm.accepts_deferred:
             hidden = ctx.ops.materialize(hidden)
         hidden, residual = self.ffn_norm.forward_residual(ctx, hidden, residual)

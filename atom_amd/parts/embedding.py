@@ -38,6 +38,27 @@ class ScaledEmbedding(TokenEmbedding):
         return ctx.ops.embedding_scaled(self.params["weight"], ids, out, self.scale)
 
 
+class PositionedEmbedding(TokenEmbedding):
+    """``table[id] + rows[position]`` as float32 rows: a learned row per position (``max_positions`` of them,
+    positions counted from 0 in each request) added to the token's row, unscaled."""
+
+    def __init__(self, vocab_size: int, hidden_size: int, max_positions: int, prefix: str = "",
+                 weight_name: str = "weight", position_name: str = "pos"):
+        super().__init__(vocab_size, hidden_size, prefix, weight_name)
+        if max_positions <= 0:
+            raise ValueError("a learned position table needs at least one row")
+        self.max_positions = int(max_positions)
+        self.position_name = position_name
+
+    def param_specs(self):
+        return {**super().param_specs(),
+                "positions": ParamSpec.single(self.position_name, (self.max_positions, self.hidden_size))}
+
+    def forward(self, ctx, ids: torch.Tensor) -> torch.Tensor:
+        out = torch.empty((ids.numel(), self.hidden_size), dtype=torch.float32, device=ids.device)
+        return ctx.ops.embedding_positions(self.params["weight"], self.params["positions"], ids, ctx.positions, out)
+
+
 class BigramEmbedding(TokenEmbedding):
     """``table[id] + pairs[(previous id * mul_prev + id * mul_cur) mod buckets]`` as float32 rows; a request's
     first token, which has no previous one, takes row ``buckets`` (the last) of ``pairs``.  The previous token of a
@@ -70,15 +91,16 @@ class BigramEmbedding(TokenEmbedding):
 
 
 class LMHead(Head):
-    """``logits = x @ W.T`` in float32 out.  ``tied_to`` names the embedding whose table it shares."""
+    """``logits = (x @ W.T) * scale`` in float32 out.  ``tied_to`` names the embedding whose table it shares."""
 
     def __init__(self, vocab_size: int, hidden_size: int, tied_to: TokenEmbedding | None = None, prefix: str = "",
-                 weight_name: str = "weight"):
+                 weight_name: str = "weight", scale: float = 1.0):
         super().__init__(prefix)
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
         self.tied_to = tied_to
         self.weight_name = weight_name
+        self.scale = float(scale)     # the float32 logits are multiplied by it
 
     def param_specs(self):
         if self.tied_to is not None:
@@ -90,10 +112,12 @@ class LMHead(Head):
         return self.tied_to.params["weight"] if self.tied_to is not None else self.params["weight"]
 
     def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
-        return ctx.ops.linear(x, self.weight, None, out_dtype=torch.float32)
+        logits = ctx.ops.linear(x, self.weight, None, out_dtype=torch.float32)
+        return logits if self.scale == 1.0 else ctx.ops.scale_rows(logits, self.scale)
 
 
 EMBEDDINGS.register("token_embedding", TokenEmbedding)
 EMBEDDINGS.register("scaled_f32_embedding", ScaledEmbedding)
 EMBEDDINGS.register("bigram_embedding", BigramEmbedding)
+EMBEDDINGS.register("positioned_f32_embedding", PositionedEmbedding)
 HEADS.register("lm_head", LMHead)

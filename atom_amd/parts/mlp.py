@@ -51,4 +51,35 @@ class GatedMLP(FeedForward):
         return ops.linear(act, self.params["down.weight"], self.p("down.bias"), defer=True)
 
 
+class DenseMLP(FeedForward):
+    """``down(act(up(x)))`` without a gate; ``activation`` one of silu, relu, gelu_tanh, relu_squared (the square
+    of ReLU).  The activation is one elementwise kernel on the up product."""
+
+    accepts_deferred = True   # the input goes to the up product as it is
+
+    ACTIVATIONS = ("silu", "relu", "gelu_tanh", "relu_squared")
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "relu_squared", prefix: str = "",
+                 names: dict[str, str] | None = None, weight_suffix: str = ""):
+        super().__init__(prefix)
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"the dense feed-forward knows the activations {self.ACTIVATIONS}, got {activation!r}")
+        self.hidden_size, self.intermediate_size, self.activation = hidden_size, intermediate_size, activation
+        self.names = {"up": "up", "down": "down", **(names or {})}
+        self.weight_suffix = weight_suffix
+
+    def param_specs(self):
+        n, i, h, sfx = self.names, self.intermediate_size, self.hidden_size, self.weight_suffix
+        return {"up.weight": ParamSpec.single(f"{n['up']}{sfx}", (i, h)),
+                "down.weight": ParamSpec.single(f"{n['down']}{sfx}", (h, i))}
+
+    def forward(self, ctx, x):
+        ops = ctx.ops
+        up = ops.linear(x, self.params["up.weight"], None)
+        act = torch.empty(tuple(up.shape), dtype=up.dtype, device=up.device)
+        ops.unary_act(up, act, self.activation)
+        return ops.linear(act, self.params["down.weight"], None, defer=True)
+
+
 FEED_FORWARDS.register("gated_mlp", GatedMLP)
+FEED_FORWARDS.register("dense_mlp", DenseMLP)

@@ -225,8 +225,9 @@ class PlainKernels:
         return out
 
     def conv_silu_state(self, x, channels, taps_weight, state, cu_seqlens_q, slot_of_seq, out, max_q_len=None,
-                        bias=None, activation="silu"):
+                        bias=None, activation="silu", x_offset=0):
         taps = taps_weight.shape[1]
+        x = x[:, x_offset:]
         for b in range(slot_of_seq.numel()):
             lo, hi, slot = int(cu_seqlens_q[b]), int(cu_seqlens_q[b + 1]), int(slot_of_seq[b])
             if slot < 0:
@@ -333,8 +334,139 @@ class PlainKernels:
         return out
 
     def rmsnorm_rows(self, x, weight, eps, rows, out):
-        out.copy_((pr.rms(x[rows.long()].to(WIDE), eps) * weight.to(WIDE)).to(out.dtype))
+        src = x if rows is None else x[rows.long()]
+        out.copy_((pr.rms(src.to(WIDE), eps) * weight.to(WIDE)).to(out.dtype))
         return out
+
+    # ---- linear recurrences with a matrix state, attention without rotation, and what stands around them
+
+    def linear_scan(self, r, r_off, r_heads, k, k_off, k_heads, v, v_off, w, w_off, state, state_off, cu_seqlens_q,
+                    slot_of_seq, out, heads, dim, vdim, per_channel=True, w_bias=None, v_scale=None, bonus=None,
+                    skip=None):
+        for b in range(slot_of_seq.numel()):
+            lo, hi, slot = int(cu_seqlens_q[b]), int(cu_seqlens_q[b + 1]), int(slot_of_seq[b])
+            if slot < 0:
+                out[lo:hi] = 0
+                continue
+            n = hi - lo
+            rr = r[lo:hi, r_off:r_off + r_heads * dim].to(WIDE).reshape(n, r_heads, dim)
+            kk = k[lo:hi, k_off:k_off + k_heads * dim].to(WIDE).reshape(n, k_heads, dim)
+            vv = v[lo:hi, v_off:v_off + heads * vdim].to(WIDE).reshape(n, heads, vdim)
+            if per_channel:
+                ww = w[lo:hi, w_off:w_off + heads * dim].to(WIDE)
+                if w_bias is not None:
+                    ww = torch.exp(-torch.exp(ww + w_bias.to(WIDE)))
+                ww = ww.reshape(n, heads, dim)
+            else:
+                ww = w[lo:hi, w_off:w_off + heads].to(WIDE)[:, :, None].expand(n, heads, dim)
+            S = state[slot, state_off:state_off + heads * dim * vdim].view(heads, dim, vdim)
+            cur = S.to(WIDE)
+            res = torch.zeros(n, heads, vdim, dtype=WIDE)
+            for t in range(n):
+                for h in range(heads):
+                    rh, kh = rr[t, h // (heads // r_heads)], kk[t, h // (heads // k_heads)]
+                    vin = vv[t, h] * (v_scale[lo + t, h].to(WIDE) if v_scale is not None else 1.0)
+                    kv = torch.outer(kh, vin)
+                    if bonus is not None:
+                        res[t, h] = (cur[h] + bonus[h].to(WIDE)[:, None] * kv).T @ rh
+                        cur[h] = ww[t, h][:, None] * cur[h] + kv
+                    else:
+                        cur[h] = ww[t, h][:, None] * cur[h] + kv
+                        res[t, h] = cur[h].T @ rh
+                    if skip is not None:
+                        res[t, h] += skip[h].to(WIDE) * vv[t, h]
+            S.copy_(cur.to(S.dtype))
+            out[lo:hi] = res.reshape(n, heads * vdim).to(out.dtype)
+        return out
+
+    def token_shift(self, x, mu, mixes, state, state_off, cu_seqlens_q, slot_of_seq, token_seq):
+        width = x.shape[1]
+        mixes.zero_()
+        for b in range(slot_of_seq.numel()):
+            lo, hi, slot = int(cu_seqlens_q[b]), int(cu_seqlens_q[b + 1]), int(slot_of_seq[b])
+            if hi == lo:
+                continue
+            rows = x[lo:hi].to(WIDE)
+            kept = state[slot, state_off:state_off + width] if slot >= 0 else torch.zeros(width)
+            before = torch.cat((kept.to(WIDE)[None], rows[:-1]))
+            for s in range(mu.shape[0]):
+                mixes[s, lo:hi] = (rows + (before - rows) * mu[s].to(WIDE)).to(mixes.dtype)
+            if slot >= 0:
+                kept.copy_(rows[-1].to(kept.dtype))
+        return mixes
+
+    def step_decay(self, raw, raw_off, dt_bias, a_log, dt, decay):
+        heads = dt.shape[1]
+        step = pl.softplus(raw[:, raw_off:raw_off + heads].to(WIDE) + dt_bias.to(WIDE))
+        dt.copy_(step.to(dt.dtype))
+        decay.copy_(torch.exp(-torch.exp(a_log.to(WIDE)) * step).to(decay.dtype))
+        return dt, decay
+
+    def group_norm_gate(self, y, groups, weight, eps, out, gate=None, gate_off=0, gate_first=False):
+        tokens, width = y.shape
+        z = y.to(WIDE)
+        g = pl.silu(gate[:, gate_off:gate_off + width].to(WIDE)) if gate is not None else None
+        if g is not None and gate_first:
+            z = z * g
+        z = pr.rms(z.reshape(tokens, groups, width // groups), eps).reshape(tokens, width)
+        if weight is not None:
+            z = z * weight.to(WIDE)
+        if g is not None and not gate_first:
+            z = z * g
+        out.copy_(z.to(out.dtype))
+        return out
+
+    def qkv_plain_write(self, proj, q_out, k_cache, v_cache, positions, slots, num_heads, num_kv_heads, head_dim,
+                        value_dim, page_size, unit_norm, eps, temperature=None, write_kv=True):
+        t = proj.shape[0]
+        q, k, v = torch.split(proj.to(WIDE), [num_heads * head_dim, num_kv_heads * head_dim, num_kv_heads * value_dim],
+                              dim=-1)
+        q = q.reshape(t, num_heads, head_dim)
+        k = k.reshape(t, num_kv_heads, head_dim)
+        v = v.reshape(t, num_kv_heads, value_dim)
+        if unit_norm:
+            q, k = pr.rms(q, eps), pr.rms(k, eps)
+        if temperature is not None and temperature[0] != 0:
+            steps = torch.div(positions.long() + 1, int(temperature[1]), rounding_mode="floor").to(WIDE)
+            q = q * (1 + temperature[0] * torch.log(steps + 1))[:, None, None]
+        q_out.zero_()
+        q_out[:, :, :head_dim] = q.to(q_out.dtype)
+        if write_kv:
+            for i in range(t):
+                slot = int(slots[i])
+                if slot < 0:
+                    continue
+                page, off = divmod(slot, page_size)
+                k_cache[page, :, off, :head_dim] = k[i].to(k_cache.dtype)
+                v_cache[page, :, :value_dim, off] = v[i].to(v_cache.dtype)
+        return q_out
+
+    def narrow_heads(self, x, value_dim):
+        return x[:, :, :value_dim].reshape(x.shape[0], -1).contiguous()
+
+    def mean_of_norms(self, xs, weights, eps, out):
+        total = sum(pr.rms(x.to(WIDE), eps) * w.to(WIDE) for x, w in zip(xs, weights))
+        out.copy_((total / len(xs)).to(out.dtype))
+        return out
+
+    def embedding_positions(self, table, rows, ids, positions, out):
+        out.copy_((table[ids.long()].to(WIDE) + rows[positions.long()].to(WIDE)).to(out.dtype))
+        return out
+
+    def unary_act(self, x, out, activation):
+        z = x.to(WIDE)
+        y = {"silu": pl.silu, "relu": torch.relu, "gelu_tanh": pl.gelu_tanh, "tanh": torch.tanh,
+             "relu_squared": lambda a: torch.relu(a) ** 2}[activation](z)
+        out.copy_(y.to(out.dtype))
+        return out
+
+    def stream_add(self, stream, x, init=False):
+        stream.copy_(x.to(torch.float32) if init else (stream.to(WIDE) + x.to(WIDE)).to(torch.float32))
+        return stream
+
+    def scale_rows(self, x, scale):
+        x.mul_(scale)
+        return x
 
     def cast_rows(self, x, dtype):
         return x.to(dtype)
