@@ -302,6 +302,35 @@ def ralitar_pair(size: str) -> tuple[dict, dict]:
     return rali, qwen
 
 
+# The Leduvik side has four layers (state-space mixer, attention side by side with time mixing, sliding-window
+# attention with unit-norm heads, state-space mixer again), each with a dense squared-ReLU feed-forward, behind learned
+# position rows; the Qwen3 side four layers of the same width with a gated feed-forward of two thirds the size (the
+# same number of weights).
+
+def leduvik_pair(size: str) -> tuple[dict, dict]:
+    width, heads, ff, vocab = {
+        "1k": (1024, 8, 2816, 32768),
+        "2k": (2048, 16, 5632, 32768),
+        "4k": (4096, 32, 11264, 65536),
+    }[size]
+    ssm = {"heads": 2 * width // 64, "vdim": 64, "state": 128, "groups": 1, "conv": 4, "norm_groups": 1}
+    window = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 1.0,
+              "mask": {"size": 1024}}
+    left = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+            "q_temp": {"coef": 0.1, "every": 512}}
+    right = {"heads": width // 64, "dim": 64, "decay_rank": 64}
+    dense = {"kind": "dense", "ff": ff * 3 // 2}
+    ledu = {"architecture": "Leduvik", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "logit_scale": 1.0,
+            "max_positions": 40960,
+            "layers": [{"type": "mamba2", "mixer": ssm, "mlp": dense},
+                       {"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": dense},
+                       {"type": "attention", "mixer": window, "mlp": dense},
+                       {"type": "mamba2", "mixer": ssm, "mlp": dense}]}
+    qwen = dict(QWEN3_8B, num_hidden_layers=4, hidden_size=width, num_attention_heads=heads,
+                num_key_value_heads=max(1, heads // 4), intermediate_size=ff, vocab_size=vocab)
+    return ledu, qwen
+
+
 def run_lotorax(args) -> dict:
     """Prefill and decode throughput of Lotorax and of Qwen3 at equal size, one engine after the other."""
     return run_design(args, "lotorax", "Lotorax", lotorax_pair, args.lotorax)
@@ -310,6 +339,11 @@ def run_lotorax(args) -> dict:
 def run_ralitar(args) -> dict:
     """Prefill and decode throughput of Ralitar and of Qwen3 at equal size, one engine after the other."""
     return run_design(args, "ralitar", "Ralitar", ralitar_pair, args.ralitar)
+
+
+def run_leduvik(args) -> dict:
+    """Prefill and decode throughput of Leduvik and of Qwen3 at equal size, one engine after the other."""
+    return run_design(args, "leduvik", "Leduvik", leduvik_pair, args.leduvik)
 
 
 def run_design(args, key: str, design: str, pair, sizes: str) -> dict:
@@ -608,6 +642,9 @@ def main() -> int:
     ap.add_argument("--ralitar", type=str, default="", metavar="SIZE[,SIZE]",
                     help="the Ralitar design beside Qwen3 at equal size (1k, 2k, 4k: the width): prefill of --context "
                          "tokens and decode at --batch, four layers each")
+    ap.add_argument("--leduvik", type=str, default="", metavar="SIZE[,SIZE]",
+                    help="the Leduvik design beside Qwen3 at equal size (1k, 2k, 4k: the width): prefill of --context "
+                         "tokens and decode at --batch, four layers each")
     ap.add_argument("--budget", type=int, default=None,
                     help="the scheduler's token budget of a step (mixed: 512 + N by default, so that portions stay 512)")
     ap.add_argument("--temperature", type=float, default=0.0, help="of the decode steps' sampling (0: greedy)")
@@ -635,6 +672,9 @@ def main() -> int:
         return 0
     if args.ralitar:
         print(json.dumps(run_ralitar(args)), flush=True)
+        return 0
+    if args.leduvik:
+        print(json.dumps(run_leduvik(args)), flush=True)
         return 0
     args.shape = args.shape or "8b"
     line = run_shape(args)

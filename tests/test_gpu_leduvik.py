@@ -1,0 +1,596 @@
+"""Leduvik on the GPU: every new kernel alone against the plain implementation's function of the same mechanism
+(float32 and bfloat16 where the kernel has both), attention with a key made to stand out just inside and just
+outside a window, at page borders and far away, a token far back that only the recurrent states remember, then the
+engine on tiny models: whole prompts, token-by-token tails, portions down to two tokens, mixed batches with pages
+and slots used again, decode steps replayed from graphs, long decoding past a window, greedy generation through
+``LLMEngine``, ``bin/trace_run`` and the command line."""
+
+import math
+
+import pytest
+import torch
+
+import leduvik_tiny as lt
+import plain_leduvik as pl
+import replay
+from helpers import gpu_ops
+from atom_amd.kernels.hip import AttentionMeta
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+TOL = {torch.float32: 2e-5, torch.bfloat16: 2e-2}
+
+
+def rnd(shape, seed, scale=1.0):
+    return torch.randn(shape, generator=torch.Generator().manual_seed(seed)) * scale
+
+
+def close(got, want, dtype, what=""):
+    got, want = got.double().cpu(), want.double().cpu()
+    scale = max(1e-6, float(want.abs().max()))
+    err = float((got - want).abs().max())
+    assert err <= TOL[dtype] * scale, f"{what}: {err:.3e} > {TOL[dtype] * scale:.3e}"
+
+
+def i32(values):
+    return torch.tensor(values, dtype=torch.int32, device=DEV)
+
+
+def f32(t):
+    return t.to(torch.float32).to(DEV).contiguous()
+
+
+def _batch(lens, slots):
+    cu = [0]
+    for n in lens:
+        cu.append(cu[-1] + n)
+    seq_of = [s for s, n in enumerate(lens) for _ in range(n)]
+    return cu, i32(cu), i32(slots), i32(seq_of)
+
+
+# ------------------------------------------------------------------ embedding, small kernels
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rows_of_token_and_position(dtype):
+    ops = gpu_ops()
+    vocab, width, places = 37, 44, 90
+    table, rows = rnd((vocab, width), 1).to(dtype), rnd((places, width), 2).to(dtype)
+    ids, positions = [5, 0, 36, 5, 17], [0, 89, 3, 1, 0]
+    out = torch.empty((5, width), dtype=torch.float32, device=DEV)
+    ops.embedding_positions(table.to(DEV), rows.to(DEV), i32(ids), i32(positions), out)
+    want = pl.embed_rows(torch.tensor(ids), torch.tensor(positions), table.double(), rows.double())
+    close(out, want, torch.float32)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_activations_sums_and_constants(dtype):
+    ops = gpu_ops()
+    x = rnd((7, 53), 1, 2.0).to(dtype)
+    for name, fn in [("relu_squared", pl.relu_squared), ("tanh", torch.tanh), ("gelu_tanh", pl.gelu_tanh), ("silu", pl.silu)]:
+        out = torch.empty((7, 53), dtype=dtype, device=DEV)
+        ops.unary_act(x.to(DEV), out, name)
+        close(out, fn(x.double()), dtype, name)
+    stream = rnd((7, 53), 2)
+    s = f32(stream)
+    ops.stream_add(s, x.to(DEV))
+    close(s, stream.double() + x.double(), torch.float32, "stream += x")
+    ops.stream_add(s, x.to(DEV), init=True)
+    close(s, x.double(), torch.float32, "stream = x")
+    ops.scale_rows(s, 0.37)
+    close(s, 0.37 * x.double(), torch.float32, "constant")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("width,n", [(40, 2), (192, 3), (1000, 1), (4096, 2)])
+def test_mean_of_normed_branches(dtype, width, n):
+    ops = gpu_ops()
+    eps = 2e-5
+    xs = [(rnd((5, width), 10 + b, 0.3 + b) + 0.2).to(dtype) for b in range(n)]
+    ws = [1 + rnd((width,), 20 + b, 0.3) for b in range(n)]
+    out = torch.empty((5, width), dtype=dtype, device=DEV)
+    ops.mean_of_norms([x.to(DEV) for x in xs], [f32(w) for w in ws], eps, out)
+    want = sum(pl.rms_norm(x.double(), w.double(), eps) for x, w in zip(xs, ws)) / n
+    close(out, want, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_heads_lose_their_padding(dtype):
+    ops = gpu_ops()
+    x = rnd((9, 5, 32), 1).to(dtype)
+    got = ops.narrow_heads(x.to(DEV), 12)
+    assert torch.equal(got.cpu(), x[:, :, :12].reshape(9, 60))
+    assert torch.equal(ops.narrow_heads(x.to(DEV), 32).cpu(), x.reshape(9, 160))
+
+
+# ------------------------------------------------------------------ the previous token's input
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_mix_with_the_previous_token_across_steps(dtype):
+    """Three requests in two steps (the middle one leaves the second step out, a padding row takes its place):
+    a request's first token mixes with zeros, a later portion's first token with the last row of the portion
+    before, whatever other requests did in between."""
+    ops = gpu_ops()
+    width, off = 50, 3
+    mu = torch.sigmoid(rnd((5, width), 1))
+    state = torch.zeros((4, off + width + 2), dtype=torch.float32, device=DEV)
+    rows = {r: rnd((n, width), 5 + r).to(dtype) for r, n in ((0, 7), (1, 3), (2, 9))}
+
+    def want(x, before):
+        prev = torch.cat((before[None], x[:-1].double()))
+        return torch.stack([x.double() + (prev - x.double()) * mu[s].double() for s in range(5)])
+
+    def run(parts, slots):
+        lens = [p.shape[0] for p in parts]
+        cu, cu_d, slot_d, seq_d = _batch(lens, slots)
+        seq_d = i32([s if slots[s] >= 0 else -1 for s, n in enumerate(lens) for _ in range(n)])
+        x = torch.cat(parts).to(DEV)
+        mixes = torch.empty((5, x.shape[0], width), dtype=dtype, device=DEV)
+        ops.token_shift(x, f32(mu), mixes, state, off, cu_d, slot_d, seq_d)
+        return [mixes[:, cu[i]:cu[i + 1]] for i in range(len(parts))]
+
+    zeros = torch.zeros(width, dtype=torch.float64)
+    first = run([rows[0][:4], rows[1], rows[2][:1]], [2, 0, 3])
+    close(first[0], want(rows[0][:4], zeros), dtype, "request 0, start")
+    close(first[1], want(rows[1], zeros), dtype, "request 1, whole")
+    close(first[2], want(rows[2][:1], zeros), dtype, "request 2, one token")
+    second = run([rows[2][1:], rnd((2, width), 9).to(dtype), rows[0][4:]], [3, -1, 2])
+    close(second[0], want(rows[2][1:], rows[2][0].double()), dtype, "request 2 goes on")
+    close(second[2], want(rows[0][4:], rows[0][3].double()), dtype, "request 0 goes on")
+    assert torch.equal(state[2, off:off + width].cpu(), rows[0][-1].float())
+    assert torch.equal(state[0, off:off + width].cpu(), rows[1][-1].float()), "a request that sat out keeps its row"
+    assert float(state[:, :off].abs().max()) == 0 and float(state[:, off + width:].abs().max()) == 0
+    assert float(state[1].abs().max()) == 0
+
+
+# ------------------------------------------------------------------ the recurrences
+
+
+def test_step_sizes_and_decays():
+    ops = gpu_ops()
+    T, H = 11, 5
+    raw = rnd((T, 9 + H), 1, 4.0)
+    raw[0, 9] = 40.0                                  # softplus without a clamp: a large input is itself
+    raw[1, 9] = -30.0
+    dt_bias, a_log = rnd((H,), 2), rnd((H,), 3, 0.7)
+    dt = torch.empty((T, H), dtype=torch.float32, device=DEV)
+    decay = torch.empty((T, H), dtype=torch.float32, device=DEV)
+    ops.step_decay(f32(raw), 9, f32(dt_bias), f32(a_log), dt, decay)
+    want = pl.softplus(raw[:, 9:].double() + dt_bias.double())
+    assert float(((dt.cpu().double() - want).abs() / want).max()) < 1e-5
+    close(decay, torch.exp(-torch.exp(a_log.double()) * want), torch.float32, "decay")
+
+
+@pytest.mark.parametrize("H,K", [(5, 8), (2, 20), (6, 48), (2, 64), (1, 128), (3, 200)])
+@pytest.mark.parametrize("lens", [[37, 1, 5], [3, 70, 1]])
+def test_time_mix_recurrence_carries_its_state(H, K, lens):
+    """The bonus recurrence over three requests in two steps against the plain token-by-token form; the state of a
+    request travels in its slot, a padding request between them touches nothing."""
+    ops = gpu_ops()
+    T2 = [9, 4, 20]
+    bonus, bias = rnd((H, K), 1, 0.5), rnd((H * K,), 2) - 1.0
+    state = torch.zeros((5, 7 + H * K * K), dtype=torch.float32, device=DEV)
+    slots = [3, 0, 4]
+    carried = [torch.zeros(H, K, K, dtype=torch.float64) for _ in lens]
+    for step, step_lens in enumerate([lens, T2]):
+        T = sum(step_lens) + 2
+        r, k, v = rnd((T, H * K), 10 + step, 0.7), rnd((T, 5 + H * K), 20 + step, 0.7), rnd((T, H * K), 30 + step)
+        raw = rnd((T, H * K), 40 + step)
+        cu, cu_d, slot_d, _ = _batch(step_lens[:2] + [2] + step_lens[2:], slots[:2] + [-1] + slots[2:])
+        out = torch.empty((T, H * K), dtype=torch.float32, device=DEV)
+        ops.linear_scan(f32(r), 0, H, f32(k), 5, H, f32(v), 0, f32(raw), 0, state, 7, cu_d, slot_d, out, H, K, K,
+                        per_channel=True, w_bias=f32(bias), bonus=f32(bonus))
+        decay = torch.exp(-torch.exp(raw.double() + bias.double()))
+        for i, s in enumerate([0, 1, 3]):
+            a, b = cu[s], cu[s + 1]
+            want, carried[i] = pl.bonus_recurrence(r[a:b].double().view(-1, H, K), k[a:b, 5:].double().view(-1, H, K),
+                                                   v[a:b].double().view(-1, H, K), decay[a:b].view(-1, H, K),
+                                                   bonus.double(), carried[i])
+            close(out[a:b], want.reshape(b - a, H * K), torch.float32, f"step {step}, request {i}")
+            close(state[slots[i], 7:], carried[i].reshape(-1), torch.float32, f"state after step {step}, request {i}")
+    assert float(state[:, :7].abs().max()) == 0 and float(state[1].abs().max()) == 0 and float(state[2].abs().max()) == 0
+
+
+@pytest.mark.parametrize("H,G,N,V", [(4, 2, 5, 6), (3, 1, 20, 12), (6, 1, 32, 48), (4, 4, 64, 32), (2, 1, 128, 64), (8, 2, 16, 100)])
+def test_state_space_recurrence_carries_its_state(H, G, N, V):
+    """Step sizes on the way into the state, one decay per head, groups of heads that share B and C, the skip
+    weight on the read-out; x, B and C are columns of one array, as the convolution leaves them."""
+    ops = gpu_ops()
+    inner = H * V
+    A, D = torch.exp(rnd((H,), 1, 0.6) - 0.5), 1 + rnd((H,), 2, 0.3)
+    state = torch.zeros((3, 11 + H * N * V), dtype=torch.float32, device=DEV)
+    slots = [2, 0]
+    carried = [torch.zeros(H, N, V, dtype=torch.float64) for _ in slots]
+    for step, lens in enumerate([[45, 2], [1, 19], [70, 1]]):
+        T = sum(lens)
+        xbc = rnd((T, inner + 2 * G * N), 10 + step, 0.8)
+        dt = pl.softplus(rnd((T, H), 20 + step).double())
+        decay = torch.exp(-A.double() * dt)
+        cu, cu_d, slot_d, _ = _batch(lens, slots)
+        out = torch.empty((T, inner), dtype=torch.float32, device=DEV)
+        x_d = f32(xbc)
+        ops.linear_scan(x_d, inner + G * N, G, x_d, inner, G, x_d, 0, f32(decay), 0, state, 11, cu_d, slot_d, out, H, N, V,
+                        per_channel=False, v_scale=f32(dt), skip=f32(D))
+        for i in range(2):
+            a, b = cu[i], cu[i + 1]
+            x, B, C = torch.split(xbc[a:b].double(), [inner, G * N, G * N], dim=-1)
+            want, carried[i] = pl.state_space_recurrence(x.view(-1, H, V), B.view(-1, G, N), C.view(-1, G, N), dt[a:b],
+                                                         A.double(), D.double(), carried[i])
+            close(out[a:b], want.reshape(b - a, inner), torch.float32, f"step {step}, request {i}")
+            close(state[slots[i], 11:], carried[i].reshape(-1), torch.float32, f"state after step {step}")
+    assert float(state[1].abs().max()) == 0 and float(state[:, :11].abs().max()) == 0
+
+
+def test_a_token_far_back_stays_in_the_states():
+    """One token writes a value like no other under a key no later token has; decays near one.  400 tokens on, in a
+    later step, a read vector along that key still returns it, from both recurrences."""
+    ops = gpu_ops()
+    H, K, V, n = 2, 32, 24, 400
+    for mode in ("bonus", "space"):
+        k, r = rnd((n, H * K), 1, 0.01), rnd((n, H * K), 2, 0.01)
+        v = rnd((n, H * V), 3, 0.01)
+        k[7].zero_()
+        k[7, 5] = k[7, K + 5] = 1.0
+        v[7] = 3.0
+        r[n - 1].zero_()
+        r[n - 1, 5] = r[n - 1, K + 5] = 1.0
+        state = torch.zeros((1, H * K * V), dtype=torch.float32, device=DEV)
+        outs = []
+        for a, b in ((0, 100), (100, n - 1), (n - 1, n)):
+            cu_d, slot_d = i32([0, b - a]), i32([0])
+            out = torch.empty((b - a, H * V), dtype=torch.float32, device=DEV)
+            if mode == "bonus":
+                w = torch.full((b - a, H * K), 0.9995)
+                ops.linear_scan(f32(r[a:b]), 0, H, f32(k[a:b]), 0, H, f32(v[a:b]), 0, f32(w), 0, state, 0, cu_d, slot_d, out,
+                                H, K, V, per_channel=True, bonus=f32(torch.zeros(H, K)))
+            else:
+                w = torch.full((b - a, H), 0.9995)
+                ops.linear_scan(f32(r[a:b]), 0, H, f32(k[a:b]), 0, H, f32(v[a:b]), 0, f32(w), 0, state, 0, cu_d, slot_d, out,
+                                H, K, V, per_channel=False)
+            outs.append(out.cpu())
+        got = float(outs[-1].mean())
+        assert abs(got - 3.0 * 0.9995 ** (n - 1 - 7 - (1 if mode == "bonus" else 0))) < 0.05, (mode, got)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("groups,gw", [(1, 40), (5, 8), (3, 100), (2, 256), (1, 288), (2, 1500), (1, 4096)])
+@pytest.mark.parametrize("gate_first", [True, False])
+def test_norm_in_parts_with_a_gate(dtype, groups, gw, gate_first):
+    ops = gpu_ops()
+    T, eps, off = 6, 3e-5, 5
+    y, gate = rnd((T, groups * gw), 1, 2.0), rnd((T, off + groups * gw + 3), 2, 1.5)
+    w = 1 + rnd((groups * gw,), 3, 0.3)
+    out = torch.empty((T, groups * gw), dtype=dtype, device=DEV)
+    ops.group_norm_gate(f32(y), groups, f32(w), eps, out, gate=f32(gate), gate_off=off, gate_first=gate_first)
+    s = pl.silu(gate[:, off:off + groups * gw].double())
+    z = y.double() * s if gate_first else y.double()
+    want = pl.unit_rms(z.view(T, groups, gw), eps).reshape(T, -1) * w.double()
+    if not gate_first:
+        want = want * s
+    close(out, want, dtype)
+
+
+@pytest.mark.parametrize("taps,channels,off", [(2, 24, 7), (3, 352, 288), (4, 300, 0), (5, 20, 3)])
+def test_convolution_reads_its_columns_of_a_wider_product(taps, channels, off):
+    """x | B | C are columns ``off .. off + channels`` of the packed product; the last ``taps - 1`` inputs travel in
+    the slot and zeros stand before a request's start."""
+    ops = gpu_ops()
+    w, bias = rnd((channels, taps), 1, 0.5), rnd((channels,), 2, 0.3)
+    state = torch.zeros((3, (taps - 1) * channels + 4), dtype=torch.float32, device=DEV)
+    slots = [1, 2]
+    before = [None, None]
+    for step, lens in enumerate([[9, 1], [1, 70], [2, 3]]):
+        T = sum(lens)
+        x = rnd((T, off + channels + 2), 10 + step)
+        cu, cu_d, slot_d, _ = _batch(lens, slots)
+        out = torch.empty((T, channels), dtype=torch.float32, device=DEV)
+        ops.conv_silu_state(f32(x), channels, f32(w), state, cu_d, slot_d, out, max_q_len=max(lens), bias=f32(bias),
+                            activation="silu", x_offset=off)
+        for i in range(2):
+            a, b = cu[i], cu[i + 1]
+            y, before[i] = pl.short_convolution(x[a:b, off:off + channels].double(), w.double(), bias.double(), before[i])
+            close(out[a:b], pl.silu(y), torch.float32, f"step {step}, request {i}")
+    assert float(state[0].abs().max()) == 0
+
+
+# ------------------------------------------------------------------ attention without rotation
+
+
+def _paged(keys, values, page, dtype, order_seed=0):
+    """Keys and values [n, G, DP] of one request in pages handed out in a shuffled order."""
+    n, G, D = keys.shape
+    pages = -(-n // page)
+    order = torch.randperm(pages + 3, generator=torch.Generator().manual_seed(order_seed))[:pages].tolist()
+    return (torch.zeros((pages + 3, G, page, D), dtype=dtype, device=DEV),
+            torch.zeros((pages + 3, G, D, page), dtype=dtype, device=DEV), order)
+
+
+def _meta(ops, dtype, T, H, G, DP, page, q_positions, ctx, order):
+    meta = AttentionMeta(token_seq=i32([0] * T), positions=i32(q_positions), block_tables=i32([order]),
+                         cu_seqlens_q=i32([0, T]), context_lens=i32([ctx]), num_seqs=1, num_tokens=T, max_q_len=T,
+                         max_context_len=ctx, page_size=page, num_prefill=1 if T > 1 else 0)
+    if T > 1:
+        short, tall = ops.attention_tile_rows(dtype, DP, page, H // G, T)
+        if short:
+            meta.rows_per_tile = short
+            meta.prefill_tiles = i32([[0, r] for r in range(0, T, short)])
+        if tall:
+            meta.tiles_by_rows = {tall: i32([[0, r] for r in range(0, T, tall)])}
+    return meta
+
+
+def _write_and_attend(ops, proj, caches, order, page, a, b, H, G, D, V, DP, dtype, unit, eps, temp, scale, window):
+    """Tokens a .. b - 1 of one request: q, k, v from the packed product to q and the pages, then attention."""
+    k_cache, v_cache = caches
+    T = b - a
+    positions = list(range(a, b))
+    slots = i32([order[p // page] * page + p % page for p in positions])
+    q = torch.empty((T, H, DP), dtype=dtype, device=DEV)
+    ops.qkv_plain_write(f32(proj[a:b]), q, k_cache, v_cache, i32(positions), slots, H, G, D, V, page, unit, eps,
+                        temperature=temp)
+    out = torch.empty((T, H, DP), dtype=dtype, device=DEV)
+    ops.paged_attention(q, k_cache, v_cache, out, _meta(ops, dtype, T, H, G, DP, page, positions, b, order), scale, window)
+    assert float(out[:, :, V:].abs().max()) == 0 if DP > V else True
+    return ops.narrow_heads(out, V)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,G,D,V,DP,page,window,unit,temp", [
+    (4, 2, 10, 6, 16, 4, 9, True, None), (6, 3, 6, 10, 16, 16, None, False, (0.25, 7)),
+    (4, 1, 64, 128, 128, 16, None, False, (0.3, 64)), (6, 2, 64, 64, 64, 16, 72, True, None),
+    (3, 3, 24, 40, 64, 8, 16, True, (0.5, 5)), (2, 1, 128, 32, 128, 16, 200, False, None)])
+def test_attention_with_unit_heads_temperature_and_window(dtype, H, G, D, V, DP, page, window, unit, temp):
+    """A whole prompt, a portion behind cached keys and single tokens against the plain attention over the same
+    (rounded) packed product; heads narrower than the pages' head size are padded with zeros."""
+    ops = gpu_ops()
+    n = (3 * window + 5) if window else 150
+    eps, scale = 2e-5, 1.3 / math.sqrt(D)
+    proj = rnd((n, 3 + H * D + G * D + G * V), 1)[:, 3:].contiguous()
+    q, k, v = torch.split(proj.double(), [H * D, G * D, G * V], dim=-1)
+    q, k, v = q.view(n, H, D), k.view(n, G, D), v.view(n, G, V)
+    if unit:
+        q, k = pl.unit_rms(q, eps), pl.unit_rms(k, eps)
+    if temp:
+        q = q * pl.query_temperature(torch.arange(n), temp[0], temp[1])[:, None, None]
+    if dtype == torch.bfloat16:
+        q, k, v = (t.to(dtype).double() for t in (q, k, v))
+    want = pl.softmax_attention(q, k, v, torch.arange(n), torch.arange(n), scale, window).reshape(n, H * V)
+    k_cache, v_cache, order = _paged(torch.zeros(n, G, DP), None, page, dtype)
+    args = (H, G, D, V, DP, dtype, unit, eps, temp, scale, window)
+    whole = _write_and_attend(ops, proj, (k_cache, v_cache), order, page, 0, n, *args)
+    close(whole, want, dtype, "whole prompt")
+    cut = n // 2 + 3
+    k_cache.zero_(), v_cache.zero_()
+    _write_and_attend(ops, proj, (k_cache, v_cache), order, page, 0, cut, *args)
+    part = _write_and_attend(ops, proj, (k_cache, v_cache), order, page, cut, n - 8, *args)
+    close(part, want[cut:n - 8], dtype, "a portion behind cached keys")
+    for pos in range(n - 8, n):
+        one = _write_and_attend(ops, proj, (k_cache, v_cache), order, page, pos, pos + 1, *args)
+        close(one[0], want[pos], dtype, f"single token at {pos}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("D,V,DP,page,window", [(64, 64, 64, 16, 72), (10, 6, 16, 4, 9), (32, 128, 128, 16, 16), (64, 32, 64, 16, 200)])
+def test_a_key_that_stands_out_is_seen_inside_the_window_only(dtype, D, V, DP, page, window):
+    """One key among hundreds has a score far above the rest and a value like no other.  The query ``window - 1``
+    places after it still returns its value, the next one does not; in prompts and for single tokens; the key right
+    before and right after a page border, at the request's first position and further on."""
+    ops = gpu_ops()
+    H = G = 2
+    n = 3 * window + 2 * page
+    for spot in (0, page - 1, page, 2 * page + 1, window + page):
+        proj = rnd((n, H * D + G * D + G * V), 4, 0.05)
+        proj[:, 3:H * D:D] = 1.0                               # every query head looks along entry 3
+        proj[spot, H * D:H * D + G * D] = 0.0
+        proj[spot, H * D + 3:H * D + G * D:D] = 40.0            # and only this key lies there
+        proj[spot, H * D + G * D:] = 7.0
+        k_cache, v_cache, order = _paged(torch.zeros(n, G, DP), None, page, dtype, order_seed=spot)
+        args = (H, G, D, V, DP, dtype, False, 1e-6, None, 1.0, window)
+        whole = _write_and_attend(ops, proj, (k_cache, v_cache), order, page, 0, n, *args).float().cpu()
+        for pos in range(n):
+            inside = spot <= pos < spot + window
+            got = float(whole[pos].mean())
+            assert (abs(got - 7.0) < 0.1) == inside, f"key at {spot}, query at {pos}: {got:.3f}"
+        for pos in (spot, spot + window - 1, spot + window, min(n - 1, spot + 2 * window)):
+            one = _write_and_attend(ops, proj, (k_cache, v_cache), order, page, pos, pos + 1, *args)
+            assert (abs(float(one.float().mean()) - 7.0) < 0.1) == (spot <= pos < spot + window), \
+                f"decoded: key at {spot}, query at {pos}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_far_key_is_found_without_a_window(dtype):
+    """Causal attention over everything: the key at position 2 of 900 is what the last query returns, decoded too."""
+    ops = gpu_ops()
+    H, G, D, V, DP, page, n = 4, 1, 64, 128, 128, 16, 900
+    proj = rnd((n, H * D + G * D + G * V), 4, 0.05)
+    proj[:, 9:H * D:D] = 0.0                                   # no other query looks along entry 9
+    proj[n - 1, :H * D] = 0.0
+    proj[n - 1, 9:H * D:D] = 1.0
+    proj[2, H * D:H * D + D] = 0.0
+    proj[2, H * D + 9] = 60.0
+    proj[2, H * D + D:] = -5.0
+    k_cache, v_cache, order = _paged(torch.zeros(n, G, DP), None, page, dtype, order_seed=3)
+    args = (H, G, D, V, DP, dtype, False, 1e-6, (0.3, 64), 1.0, None)
+    whole = _write_and_attend(ops, proj, (k_cache, v_cache), order, page, 0, n, *args)
+    assert abs(float(whole[n - 1].float().mean()) + 5.0) < 0.1 and abs(float(whole[n - 2].float().mean())) < 1.0
+    one = _write_and_attend(ops, proj, (k_cache, v_cache), order, page, n - 1, n, *args)
+    assert abs(float(one.float().mean()) + 5.0) < 0.1
+
+
+# ------------------------------------------------------------------ the engine
+
+LENGTHS = {"A": [1, 7, 33, 150, 64, 300], "B": [2, 19, 45, 260, 128], "C": [3, 40, 17, 270, 96, 161],
+           "X": [5, 40, 130, 300]}
+# float32: every position against the largest logit of its request; where the plain implementation in float32 is
+# itself further from float64 than that, four times its own distance is allowed
+F32_TOL = dict(max=1e-4, mean=2e-5)
+BF16_TOL = dict(max=6e-2, mean=1.2e-2)
+
+
+def _requests(which, seed=0):
+    return {f"r{k}": lt.ids(which, n, seed * 100 + k) for k, n in enumerate(LENGTHS[which])}
+
+
+def _check(steps, results, requests, which, dtype, what):
+    rows = replay.collect(steps, results)
+    over, judged = [], 0
+    for rid, tokens in requests.items():
+        want = lt.oracle(which, tokens)
+        scale = float(want.abs().max())
+        inherent = lt.float32_error(which, tokens) / scale if dtype == "float32" else None
+        assert len(rows[rid]) == len(tokens)
+        for pos, got in sorted(rows[rid].items()):
+            assert torch.isfinite(got).all(), f"{what} request {rid} position {pos}: not finite"
+            diff = (got.double() - want[pos]).abs()
+            worst, mean = float(diff.max()) / scale, float(diff.mean()) / scale
+            judged += 1
+            if dtype == "float32":
+                room = max(1.0, 4 * float(inherent[pos]) / F32_TOL["max"])
+                assert worst <= room * F32_TOL["max"] and mean <= room * F32_TOL["mean"], \
+                    f"{what} request {rid} position {pos}: max {worst:.3e} mean {mean:.3e} of the largest logit"
+            elif worst > BF16_TOL["max"] or mean > BF16_TOL["mean"]:
+                over.append((rid, pos, worst, mean))
+    assert len(over) <= 0.02 * judged, f"{what}: {len(over)} of {judged} over: {over[:5]}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("cut", ["whole", "tail", "portions", "mixed"])
+def test_cuts_match_plain(which, cut, dtype):
+    requests = _requests(which)
+    steps = getattr(replay, cut)(requests)
+    pages = -(-replay.peak_tokens(steps, 16) // 16)
+    core = lt.core(which, dtype, gpu_ops(), DEV, num_pages=pages, page_size=16, graph_sizes=[1, 2, 4] if cut != "whole" else None)
+    results = replay.run_in_process(core, steps)
+    _check(steps, results, requests, which, dtype, f"{which}/{cut}/{dtype}")
+    assert all(pool.num_free == pool.num_pages for pool in core.manager.pools)
+    if cut == "tail":
+        assert core.graphs is not None and core.graphs.replays >= 32, "single tokens replay captured graphs"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cut", ["whole", "mixed"])
+def test_wider_model_reaches_every_product_kernel(cut, dtype):
+    """Prompts of 5, 40, 130 and 300 tokens on a model of width 384: products of few rows, of up to 64, of up to 256
+    and the library's, with float32 outputs, all against the plain implementation."""
+    requests = _requests("X")
+    steps = getattr(replay, cut)(requests)
+    pages = -(-replay.peak_tokens(steps, 16) // 16)
+    core = lt.core("X", dtype, gpu_ops(), DEV, num_pages=pages, page_size=16, graph_sizes=[1, 2, 4] if cut != "whole" else None)
+    results = replay.run_in_process(core, steps)
+    _check(steps, results, requests, "X", dtype, f"X/{cut}/{dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_small_pages_slots_used_again_and_long_decoding(dtype):
+    """Pages of 4 tokens, two state slots for five requests, and 150 tokens decoded one by one, past the windows of
+    9 tokens many times over and past a step of the query temperature, every one of them compared."""
+    requests = {"long": lt.ids("A", 330, 1), "b": lt.ids("A", 23, 2), "c": lt.ids("A", 50, 3), "d": lt.ids("A", 9, 4),
+                "e": lt.ids("A", 31, 5)}
+    steps = replay.mixed(requests, seed=6, max_live=2, decode_tail=150)
+    pages = -(-replay.peak_tokens(steps, 4) // 4)
+    core = lt.core("A", dtype, gpu_ops(), DEV, num_pages=pages, page_size=4, max_num_seqs=2, graph_sizes=[1, 2])
+    results = replay.run_in_process(core, steps)
+    _check(steps, results, requests, "A", dtype, f"A/page4/{dtype}")
+
+
+def test_logits_do_not_depend_on_the_batch_or_the_cut():
+    """float32: a request's logits alone, cut in portions, and beside others differ by rounding of sums only."""
+    requests = _requests("C")
+    runs = []
+    for cut in ("whole", "portions", "mixed"):
+        steps = getattr(replay, cut)(requests)
+        core = lt.core("C", "float32", gpu_ops(), DEV, num_pages=80, page_size=16)
+        runs.append(replay.collect(steps, replay.run_in_process(core, steps)))
+    for rid in requests:
+        for pos in runs[0][rid]:
+            for other in runs[1:]:
+                assert float((runs[0][rid][pos] - other[rid][pos]).abs().max()) <= 2e-5 * float(runs[0][rid][pos].abs().max())
+
+
+def test_stream_after_every_run_of_a_layer():
+    """float32: the stream after each run of a layer (a repeated layer counts every time) against the plain
+    implementation's, so that a fault shows at the layer that makes it."""
+    tokens = lt.ids("A", 45, 8)
+    trail = []
+    pl.forward(lt.CONFIGS["A"], lt.tensors("A"), tokens, trail=trail)
+    core = lt.core("A", "float32", gpu_ops(), DEV, num_pages=8, page_size=16)
+    got = []
+    blocks = core.model.blocks
+    originals = [b.forward for b in blocks]
+
+    def watch(block, inner):
+        def forward(ctx, hidden, residual, cache):
+            if residual is not None:       # what stood after the run before: the stream plus its pending summand
+                got.append((residual + ctx.ops.materialize(hidden).float()).cpu())
+            return inner(ctx, hidden, residual, cache)
+        return forward
+
+    for b, inner in zip(blocks, originals):
+        b.forward = watch(b, inner)
+    try:
+        from atom_amd.engine.core import StepEntry
+        core.step([StepEntry("a", tokens, [len(tokens) - 1])])
+    finally:
+        for b, inner in zip(blocks, originals):
+            b.forward = inner
+    assert len(got) >= len(trail) - 1
+    for run, (mine, want) in enumerate(zip(got, trail)):
+        if run + 1 < len(trail) and any(r.enters for r in core.model.order[run + 1:run + 2]):
+            continue                       # the join has already added the embedding's output here
+        close(mine, want, torch.float32, f"after run {run}")
+
+
+@pytest.mark.parametrize("which,dtype", [("A", "fp32"), ("B", "fp32"), ("C", "fp32"), ("C", "bf16")])
+def test_greedy_generation_through_the_engine(which, dtype):
+    from atom_amd import LLMEngine, SamplingParams
+
+    llm = LLMEngine(lt.folder(which), dtype=dtype, ops=gpu_ops(), kv_cache_block_size=16, num_kvcache_blocks=64,
+                    max_num_seqs=4, max_num_batched_tokens=64, max_model_len=384)
+    prompts = [lt.ids(which, n, 70 + n) for n in (1, 9, 40, 130, 65)]
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True))
+    for prompt, out in zip(prompts, outs):
+        tokens = list(prompt)
+        assert len(out["token_ids"]) == 10
+        for token in out["token_ids"]:
+            logits = lt.oracle(which, tokens)[-1]
+            best = int(logits.argmax())
+            slack = 0.0 if dtype == "fp32" else 0.06 * float(logits.abs().max())
+            assert token == best or float(logits[best] - logits[token]) <= slack
+            tokens.append(token)
+    assert all(p.num_free == p.num_pages for p in llm.core.manager.pools)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_program(dtype, tmp_path):
+    requests = {k: v for k, v in list(_requests("B").items())[:4]}
+    steps = replay.mixed(requests, seed=2, max_live=3)
+    results = replay.run_program(lt.folder("B"), dtype, steps, str(tmp_path / "out"), replay.peak_tokens(steps, 64),
+                                 lt.CONFIGS["B"]["vocab"])
+    _check(steps, results, requests, "B", dtype, f"program/{dtype}")
+
+
+def test_command_line():
+    """``python -m atom_amd.examples.simple_inference`` on a Leduvik folder: the registry picks the design from
+    config.json; greedy completions are the plain implementation's."""
+    import random
+    import re
+    import subprocess
+    import sys
+
+    cmd = [sys.executable, "-m", "atom_amd.examples.simple_inference", "--model", lt.folder("B"), "--temperature", "0",
+           "--max-tokens", "6", "--block_size", "16", "--num-kvcache-blocks", "32", "--max-num-seqs", "4", "--dtype", "fp32",
+           "--max-model-len", "256", "--seed", "3"]
+    res = subprocess.run(cmd, cwd=replay.ROOT, capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr[-2000:]
+    assert res.stdout.count("Completion:") == 3 and res.stdout.count("finish_reason=max_tokens") == 3
+    rng = random.Random(3)
+    prompts = [[rng.randrange(lt.CONFIGS["B"]["vocab"]) for _ in range(n)] for n in (5, 17, 33)]
+    shown = [eval(m) for m in re.findall(r"Completion: (\[.*?\])", res.stdout)]
+    for prompt, out in zip(prompts, shown):
+        tokens = list(prompt)
+        for token in out:
+            assert token == int(lt.oracle("B", tokens)[-1].argmax())
+            tokens.append(token)
