@@ -10,10 +10,20 @@
 //       S <- diag(w) S + k v^T;        o = S^T r
 //
 // v may first be multiplied by a step size per (token, head), and o may receive skip[h] * (the unscaled v).  The
-// columns of S never meet, so a column lives in registers, spread over LPC adjacent lanes of 16 rows each; r, k and w
-// of a run of tokens are staged in LDS by all lanes at once, the decay formed on the way (as given, or
-// exp(-exp(x + bias))).  A block is one wave: it owns 64 / LPC columns of one head of one request and walks the
-// request's tokens of this step in order, so a token's result depends on its own request only.
+// columns of S never meet, so a column lives in registers, spread over LPC adjacent lanes of 16 rows each.  A wave
+// owns 64 / LPC columns of one head; the waves of a block (up to four) own neighbouring columns and share what they
+// stage in LDS for 16 tokens at a time: r, k and the decays (formed on the way: as given, or exp(-exp(x + bias))),
+// the block's columns of v and the step sizes.
+//
+// Requests that bring no more than a run's length of tokens are walked by one block per (request, head, columns):
+// the state comes from the slot and goes back there.  Longer requests are cut into runs that are worked side by
+// side, which the recurrence allows because a run acts on the state as S -> diag(a) S + B:
+//   1. every run but a request's last forms B (its tokens applied to a zero state) and a (the product of its decays);
+//   2. per request the state before each run is folded from the slot's state through the runs ahead of it;
+//   3. every run walks its tokens again from that state and writes the outputs; the last run leaves the state in
+//      the slot.
+// Run j of request s (tokens from t0) has the scratch place t0 / R + s + j, which no other run has.  A token's
+// result depends on its own request only; cutting a request differently changes the order of roundings, no more.
 //
 // Around it: token_shift (a token's input mixed with the previous token's, the previous token kept per request),
 // step_decay (softplus step sizes and the decays exp(-exp(A_log) dt) of a state-space layer), group_norm_gate (RMS
@@ -21,7 +31,8 @@
 #include "common.h"
 
 constexpr int kScanRows = 16;    // rows of S a lane holds
-constexpr int kScanRun = 16;     // tokens staged at a time
+constexpr int kScanStage = 16;   // tokens staged at a time
+constexpr int kScanWaves = 4;    // the most waves of a block
 
 struct ScanArgs {
   const float* r; long ldr; int r_div;       // head h reads r-head h / r_div, K entries each
@@ -35,85 +46,202 @@ struct ScanArgs {
   float* out; long ldo;                      // [T, H * V]
   float* state; long slot_stride; long state_off;
   const int* cu_seqlens; const int* slot_of_seq;
-  int H, K, V, lpc;
+  int num_seqs, H, K, V, lpc, waves;
+  int run_len;                               // R, a multiple of kScanStage; 0: a request is one run whatever its length
+  float* run_state;                          // [places, H, K, V]: B of a run after pass 1, the state before it after pass 2
+  float* run_decay;                          // [places, H, K]: the product of a run's decays
 };
 
-__global__ void __launch_bounds__(64) linear_scan_kernel(ScanArgs a) {
-  extern __shared__ float staged[];          // [kScanRun][3][KP]: r, k, w of a run's tokens
-  const int seq = blockIdx.x, h = blockIdx.y;
+// Which request and which of its runs the block with index b works on: the last s with cu[s] / R + s <= b.
+__device__ __forceinline__ bool scan_place(const ScanArgs& a, int b, int& seq, int& run, int& runs) {
+  if (a.run_len == 0) {
+    seq = b; run = 0; runs = 1;
+    return true;
+  }
+  int lo = 0, hi = a.num_seqs - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (a.cu_seqlens[mid] / a.run_len + mid <= b) lo = mid; else hi = mid - 1;
+  }
+  seq = lo;
+  const int t0 = a.cu_seqlens[seq], len = a.cu_seqlens[seq + 1] - t0;
+  runs = max(1, (len + a.run_len - 1) / a.run_len);
+  run = b - (t0 / a.run_len + seq);
+  return run >= 0 && run < runs;
+}
+
+// PASS 0: a run with outputs (the whole request, or pass 3 of a long one); PASS 1: B and a of a run, no outputs.
+template <int PASS>
+__global__ void __launch_bounds__(64 * kScanWaves) linear_scan_kernel(ScanArgs a) {
+  extern __shared__ float staged[];          // [kScanStage][3 * KP + VW + 1, padded]: r, k, w, the block's v columns, step size
+  const int h = blockIdx.y;
   const int lpc = a.lpc, cols = kWave / lpc;
   const int KP = lpc * kScanRows;
-  const int lane = threadIdx.x;
-  const int col = blockIdx.z * cols + lane / lpc;
+  const int VW = a.waves * cols;             // columns of v the block owns
+  const int per_token = 3 * KP + ((VW + 4) & ~3);   // a token's rows stay 16-byte aligned
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int col0 = blockIdx.z * VW;
+  const int vcol = wave * cols + lane / lpc; // the lane's column among the block's
+  const int col = col0 + vcol;
   const int part = lane % lpc;               // which 16 rows of the column
   const int row0 = part * kScanRows;
-  const int t0 = a.cu_seqlens[seq], t1 = a.cu_seqlens[seq + 1];
-  const int slot = a.slot_of_seq[seq];
-  const bool live = col < a.V;
   const int K = a.K, V = a.V;
+  int seq, run, runs;
+  if (!scan_place(a, blockIdx.x, seq, run, runs)) return;
+  if (PASS == 1 && run == runs - 1) return;  // nothing follows a request's last run
+  const int s0 = a.cu_seqlens[seq], s1 = a.cu_seqlens[seq + 1];
+  const int t0 = a.run_len == 0 ? s0 : s0 + run * a.run_len;
+  const int t1 = a.run_len == 0 ? s1 : min(s1, t0 + a.run_len);
+  const int slot = a.slot_of_seq[seq];
+  const bool live = col < V;
   if (slot < 0) {                            // a padding row: nothing to carry, its output is never read
-    for (int t = t0; t < t1; ++t)
-      if (live && part == 0) a.out[(size_t)t * a.ldo + (size_t)h * V + col] = 0.f;
+    if (PASS == 0)
+      for (int t = t0; t < t1; ++t)
+        if (live && part == 0) a.out[(size_t)t * a.ldo + (size_t)h * V + col] = 0.f;
     return;
   }
-  float* S_mem = a.state + (size_t)slot * a.slot_stride + a.state_off + (size_t)h * K * V;
+  const size_t place = a.run_len == 0 ? 0 : (size_t)(s0 / a.run_len + seq + run);
+  float* S_slot = a.state + (size_t)slot * a.slot_stride + a.state_off + (size_t)h * K * V;
+  float* S_run = a.run_state != nullptr ? a.run_state + (place * a.H + h) * (size_t)K * V : nullptr;
   float S[kScanRows];
+  if (PASS == 1) {
 #pragma unroll
-  for (int i = 0; i < kScanRows; ++i) S[i] = (live && row0 + i < K) ? S_mem[(size_t)(row0 + i) * V + col] : 0.f;
-  float u[kScanRows];
+    for (int i = 0; i < kScanRows; ++i) S[i] = 0.f;
+  } else {
+    const float* from = runs > 1 ? S_run : S_slot;
+#pragma unroll
+    for (int i = 0; i < kScanRows; ++i) S[i] = (live && row0 + i < K) ? from[(size_t)(row0 + i) * V + col] : 0.f;
+  }
+  float u[kScanRows];                        // PASS 0: the bonus; PASS 1: the product of the run's decays
   const bool before = a.bonus != nullptr;
 #pragma unroll
-  for (int i = 0; i < kScanRows; ++i) u[i] = (before && row0 + i < K) ? a.bonus[(size_t)h * K + row0 + i] : 0.f;
+  for (int i = 0; i < kScanRows; ++i)
+    u[i] = PASS == 1 ? 1.f : ((before && row0 + i < K) ? a.bonus[(size_t)h * K + row0 + i] : 0.f);
   const float skip = a.skip != nullptr ? a.skip[h] : 0.f;
   const int rh = h / a.r_div, kh = h / a.k_div;
 
-  for (int base = t0; base < t1; base += kScanRun) {
-    const int n = min(kScanRun, t1 - base);
+  for (int base = t0; base < t1; base += kScanStage) {
+    const int n = min(kScanStage, t1 - base);
     __syncthreads();
-    for (int e = lane; e < n * KP; e += kWave) {
+    for (int e = tid; e < n * KP; e += blockDim.x) {
       const int j = e / KP, i = e - j * KP;
       const size_t t = (size_t)(base + j);
       float rv = 0.f, kv = 0.f, wv = 1.f;
       if (i < K) {
-        rv = a.r[t * a.ldr + (size_t)rh * K + i];
+        if (PASS == 0) rv = a.r[t * a.ldr + (size_t)rh * K + i];
         kv = a.k[t * a.ldk + (size_t)kh * K + i];
         wv = a.w_per_channel ? a.w[t * a.ldw + (size_t)h * K + i] : a.w[t * a.ldw + h];
         if (a.w_mode == 1) wv = expf(-expf(wv + a.w_bias[(size_t)h * K + i]));
       }
-      float* dst = staged + (size_t)j * 3 * KP;
+      float* dst = staged + (size_t)j * per_token;
       dst[i] = rv;
       dst[KP + i] = kv;
       dst[2 * KP + i] = wv;
     }
+    for (int e = tid; e < n * (VW + 1); e += blockDim.x) {
+      const int j = e / (VW + 1), c = e - j * (VW + 1);
+      const size_t t = (size_t)(base + j);
+      float x;
+      if (c == VW) x = a.v_scale != nullptr ? a.v_scale[t * a.ldvs + h] : 1.f;
+      else x = col0 + c < V ? a.v[t * a.ldv + (size_t)h * V + col0 + c] : 0.f;
+      staged[(size_t)j * per_token + 3 * KP + c] = x;
+    }
     __syncthreads();
     for (int j = 0; j < n; ++j) {
-      const size_t t = (size_t)(base + j);
-      const float* src = staged + (size_t)j * 3 * KP + row0;
-      const float v_raw = live ? a.v[t * a.ldv + (size_t)h * V + col] : 0.f;
-      const float v = a.v_scale != nullptr ? v_raw * a.v_scale[t * a.ldvs + h] : v_raw;
+      const float* src = staged + (size_t)j * per_token;
+      const float4* r4 = reinterpret_cast<const float4*>(src + row0);
+      const float4* k4 = reinterpret_cast<const float4*>(src + KP + row0);
+      const float4* w4 = reinterpret_cast<const float4*>(src + 2 * KP + row0);
+      const float v_raw = src[3 * KP + vcol];
+      const float v = v_raw * src[3 * KP + VW];
       float acc = 0.f;
-      if (before) {
 #pragma unroll
-        for (int i = 0; i < kScanRows; ++i) {
-          const float kv = src[KP + i] * v;
-          acc += src[i] * (S[i] + u[i] * kv);
-          S[i] = src[2 * KP + i] * S[i] + kv;
-        }
-      } else {
+      for (int q = 0; q < kScanRows / 4; ++q) {
+        const float4 kq = k4[q], wq = w4[q];
+        const float kk[4] = {kq.x, kq.y, kq.z, kq.w}, ww[4] = {wq.x, wq.y, wq.z, wq.w};
+        if (PASS == 1) {
 #pragma unroll
-        for (int i = 0; i < kScanRows; ++i) {
-          S[i] = src[2 * KP + i] * S[i] + src[KP + i] * v;
-          acc += src[i] * S[i];
+          for (int c = 0; c < 4; ++c) {
+            S[4 * q + c] = ww[c] * S[4 * q + c] + kk[c] * v;
+            u[4 * q + c] *= ww[c];
+          }
+        } else {
+          const float4 rq = r4[q];
+          const float rr[4] = {rq.x, rq.y, rq.z, rq.w};
+          if (before) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+              const float kv = kk[c] * v;
+              acc += rr[c] * (S[4 * q + c] + u[4 * q + c] * kv);
+              S[4 * q + c] = ww[c] * S[4 * q + c] + kv;
+            }
+          } else {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+              S[4 * q + c] = ww[c] * S[4 * q + c] + kk[c] * v;
+              acc += rr[c] * S[4 * q + c];
+            }
+          }
         }
       }
-      for (int off = lpc >> 1; off > 0; off >>= 1) acc += __shfl_xor(acc, off, kWave);
-      if (live && part == 0) a.out[t * a.ldo + (size_t)h * V + col] = acc + skip * v_raw;
+      if (PASS == 0) {
+        for (int off = lpc >> 1; off > 0; off >>= 1) acc += __shfl_xor(acc, off, kWave);
+        if (live && part == 0) a.out[(size_t)(base + j) * a.ldo + (size_t)h * V + col] = acc + skip * v_raw;
+      }
     }
   }
-  if (live) {
+  if (PASS == 1) {
+    if (live) {
+#pragma unroll
+      for (int i = 0; i < kScanRows; ++i)
+        if (row0 + i < K) S_run[(size_t)(row0 + i) * V + col] = S[i];
+    }
+    if (col == 0) {
+      float* decay = a.run_decay + (place * a.H + h) * (size_t)K;
+#pragma unroll
+      for (int i = 0; i < kScanRows; ++i)
+        if (row0 + i < K) decay[row0 + i] = u[i];
+    }
+  } else if (live && run == runs - 1) {
 #pragma unroll
     for (int i = 0; i < kScanRows; ++i)
-      if (row0 + i < K) S_mem[(size_t)(row0 + i) * V + col] = S[i];
+      if (row0 + i < K) S_slot[(size_t)(row0 + i) * V + col] = S[i];
+  }
+}
+
+// Pass 2: per request of several runs and per entry of S, the state before every run: the slot's state before the
+// first, then S <- a_j S + B_j from run to run; it takes B's place.
+__global__ void __launch_bounds__(256) linear_scan_fold_kernel(ScanArgs a) {
+  const int seq = blockIdx.x, h = blockIdx.y;
+  const int K = a.K, V = a.V;
+  const int e = blockIdx.z * blockDim.x + threadIdx.x;
+  if (e >= K * V) return;
+  const int slot = a.slot_of_seq[seq];
+  const int t0 = a.cu_seqlens[seq], len = a.cu_seqlens[seq + 1] - t0;
+  const int runs = (len + a.run_len - 1) / a.run_len;
+  if (slot < 0 || runs <= 1) return;
+  const int row = e / V;
+  const size_t first = (size_t)(t0 / a.run_len + seq);
+  const size_t stride = (size_t)a.H * K * V, dstride = (size_t)a.H * K;
+  float* B = a.run_state + (first * a.H + h) * (size_t)K * V + e;
+  const float* decay = a.run_decay + (first * a.H + h) * (size_t)K + row;
+  float S = a.state[(size_t)slot * a.slot_stride + a.state_off + (size_t)h * K * V + e];
+  constexpr int kAhead = 8;
+  for (int j0 = 0; j0 < runs; j0 += kAhead) {
+    float b[kAhead], d[kAhead];
+#pragma unroll
+    for (int c = 0; c < kAhead; ++c) {
+      const bool has = j0 + c < runs - 1;
+      b[c] = has ? B[(size_t)(j0 + c) * stride] : 0.f;
+      d[c] = has ? decay[(size_t)(j0 + c) * dstride] : 0.f;
+    }
+#pragma unroll
+    for (int c = 0; c < kAhead; ++c) {
+      if (j0 + c < runs) {
+        B[(size_t)(j0 + c) * stride] = S;
+        S = d[c] * S + b[c];
+      }
+    }
   }
 }
 
@@ -121,23 +249,36 @@ ATOM_EXPORT int atom_linear_scan(const float* r, long ldr, int r_div, const floa
                                  long ldv, const float* w, long ldw, int w_per_channel, const float* w_bias, int w_mode,
                                  const float* v_scale, long ldvs, const float* bonus, const float* skip, float* out,
                                  long ldo, float* state, long slot_stride, long state_off, const int* cu_seqlens,
-                                 const int* slot_of_seq, int num_seqs, int H, int K, int V, hipStream_t stream) {
-  if (H <= 0 || K <= 0 || V <= 0 || num_seqs < 0 || r_div <= 0 || k_div <= 0) return ATOM_BAD_SHAPE;
+                                 const int* slot_of_seq, int num_seqs, int H, int K, int V, int tokens, int run_len,
+                                 float* run_state, float* run_decay, long places, hipStream_t stream) {
+  if (H <= 0 || K <= 0 || V <= 0 || num_seqs < 0 || r_div <= 0 || k_div <= 0 || tokens < 0) return ATOM_BAD_SHAPE;
   if (r == nullptr || k == nullptr || v == nullptr || w == nullptr || out == nullptr || state == nullptr) return ATOM_BAD_SHAPE;
   if (cu_seqlens == nullptr || slot_of_seq == nullptr) return ATOM_BAD_SHAPE;
   if (w_mode != 0 && w_mode != 1) return ATOM_UNSUPPORTED;
   if (w_mode == 1 && (w_bias == nullptr || !w_per_channel)) return ATOM_BAD_SHAPE;
   if (state_off < 0 || slot_stride < state_off + (long)H * K * V) return ATOM_BAD_SHAPE;
   if (K > 16 * kScanRows) return ATOM_TOO_LARGE;
+  if (run_len < 0 || run_len % kScanStage) return ATOM_BAD_SHAPE;
+  const long need = run_len > 0 ? (long)(tokens + run_len - 1) / run_len + num_seqs : 0;
+  if (run_len > 0 && (run_state == nullptr || run_decay == nullptr || places < need)) return ATOM_BAD_SHAPE;
   if (num_seqs == 0) return ATOM_OK;
   int lpc = 1;
   while (lpc * kScanRows < K) lpc <<= 1;
   const int cols = kWave / lpc;
-  if (num_seqs > 0x7fffffff / 1 || H > 65535 || (V + cols - 1) / cols > 65535) return ATOM_TOO_LARGE;
+  const int waves = min(kScanWaves, (V + cols - 1) / cols);
+  const int vw = waves * cols;
+  const long blocks_x = run_len > 0 ? need : num_seqs;
+  if (blocks_x > 0x7fffffff || H > 65535 || (V + vw - 1) / vw > 65535 || ((long)K * V + 255) / 256 > 65535) return ATOM_TOO_LARGE;
   ScanArgs a{r, ldr, r_div, k, ldk, k_div, v, ldv, w, ldw, w_per_channel, w_bias, w_mode, v_scale, ldvs, bonus, skip,
-             out, ldo, state, slot_stride, state_off, cu_seqlens, slot_of_seq, H, K, V, lpc};
-  const size_t smem = (size_t)kScanRun * 3 * lpc * kScanRows * sizeof(float);
-  hipLaunchKernelGGL(linear_scan_kernel, dim3(num_seqs, H, (V + cols - 1) / cols), dim3(kWave), smem, stream, a);
+             out, ldo, state, slot_stride, state_off, cu_seqlens, slot_of_seq, num_seqs, H, K, V, lpc, waves, run_len,
+             run_len > 0 ? run_state : nullptr, run_len > 0 ? run_decay : nullptr};
+  const size_t smem = (size_t)kScanStage * (3 * lpc * kScanRows + ((vw + 4) & ~3)) * sizeof(float);
+  const dim3 grid((unsigned)blocks_x, H, (V + vw - 1) / vw), block(kWave * waves);
+  if (run_len > 0) {
+    hipLaunchKernelGGL(linear_scan_kernel<1>, grid, block, smem, stream, a);
+    hipLaunchKernelGGL(linear_scan_fold_kernel, dim3(num_seqs, H, (unsigned)(((long)K * V + 255) / 256)), dim3(256), 0, stream, a);
+  }
+  hipLaunchKernelGGL(linear_scan_kernel<0>, grid, block, smem, stream, a);
   return launch_status();
 }
 

@@ -1160,9 +1160,12 @@ class HipKernels:
     def _at(t: torch.Tensor, offset: int):
         return ctypes.c_void_p(t.data_ptr() + t.element_size() * offset)
 
+    SCAN_RUN = 64     # tokens of a run of the linear recurrences (a multiple of 16)
+
     def linear_scan(self, r, r_off: int, r_heads: int, k, k_off: int, k_heads: int, v, v_off: int, w, w_off: int,
                     state, state_off: int, cu_seqlens_q, slot_of_seq, out, heads: int, dim: int, vdim: int,
-                    per_channel: bool = True, w_bias=None, v_scale=None, bonus=None, skip=None):
+                    per_channel: bool = True, w_bias=None, v_scale=None, bonus=None, skip=None,
+                    max_q_len: int | None = None):
         """A linear recurrence with a state of ``dim`` x ``vdim`` per head over each request's tokens:
         ``S <- diag(w) S + k v^T`` with the read-out ``o = (S_before + diag(bonus) k v^T)^T r`` where ``bonus``
         [heads, dim] is given, else ``o = S_after^T r``.  All inputs float32 [tokens, *], read from a column offset:
@@ -1171,7 +1174,9 @@ class HipKernels:
         ``per_channel`` and else one per head; with ``w_bias`` [heads, dim] the decay is ``exp(-exp(w + w_bias))``.
         ``v_scale`` [tokens, heads] multiplies v on its way into the state; ``skip`` [heads] adds ``skip * v`` (v as
         given) to the read-out.  The heads' matrices [heads, dim, vdim] start at ``state_off`` of a slot's row of
-        ``state``; requests with slot -1 are padding.  ``out`` float32 [tokens, heads * vdim]."""
+        ``state``; requests with slot -1 are padding.  ``out`` float32 [tokens, heads * vdim].  ``max_q_len``: the most tokens a
+        request brings (an upper bound; default: all tokens); beyond ``SCAN_RUN`` tokens requests are cut into runs of
+        that length that are worked side by side, through scratch memory of a state per run."""
         tokens = out.shape[0]
         seqs = slot_of_seq.numel()
         if heads % r_heads or heads % k_heads:
@@ -1194,12 +1199,19 @@ class HipKernels:
         if skip is not None:
             self._check("skip", skip, torch.float32, (heads,))
         L = ctypes.c_long
+        longest = tokens if max_q_len is None else min(tokens, max_q_len)
+        run_len, places, run_state, run_decay = 0, 0, None, None
+        if longest > self.SCAN_RUN:
+            run_len = self.SCAN_RUN
+            places = -(-tokens // run_len) + seqs
+            run_state = torch.empty((places, heads, dim, vdim), dtype=torch.float32, device=out.device)
+            run_decay = torch.empty((places, heads, dim), dtype=torch.float32, device=out.device)
         self._done("linear_scan", self.lib.atom_linear_scan(
             self._at(r, r_off), L(r.shape[1]), heads // r_heads, self._at(k, k_off), L(k.shape[1]), heads // k_heads,
             self._at(v, v_off), L(v.shape[1]), self._at(w, w_off), L(w.shape[1]), int(bool(per_channel)), _ptr(w_bias),
             1 if w_bias is not None else 0, _ptr(v_scale), L(heads), _ptr(bonus), _ptr(skip), _ptr(out),
             L(heads * vdim), _ptr(state), L(state.shape[1]), L(state_off), _ptr(cu_seqlens_q), _ptr(slot_of_seq), seqs,
-            heads, dim, vdim, self._stream()))
+            heads, dim, vdim, tokens, run_len, _ptr(run_state), _ptr(run_decay), L(places), self._stream()))
         return out
 
     def token_shift(self, x, mu, mixes, state, state_off: int, cu_seqlens_q, slot_of_seq, token_seq):

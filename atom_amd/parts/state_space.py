@@ -82,7 +82,7 @@ class StateSpaceMixer(Mixer):
         y = torch.empty((T, inner), dtype=torch.float32, device=x.device)
         ops.linear_scan(xbc, inner + G * N, G, xbc, inner, G, xbc, 0, decay, 0, cache.state, self.conv_floats,
                         ctx.cu_seqlens_q, ctx.slot_of_seq, y, H, N, V, per_channel=False, v_scale=dt,
-                        skip=self.params["D"])
+                        skip=self.params["D"], max_q_len=ctx.max_q_len)
         out = torch.empty((T, inner), dtype=x.dtype, device=x.device)
         ops.group_norm_gate(y, self.norm_groups, self.params["norm.weight"], self.norm_eps, out, gate=proj, gate_off=0,
                             gate_first=True)

@@ -86,7 +86,8 @@ class TimeMixRecurrence(Mixer):
                        exact=True)
         o = torch.empty((T, c), dtype=torch.float32, device=x.device)
         ops.linear_scan(r, 0, H, k, 0, H, v, 0, raw, 0, cache.state, W, ctx.cu_seqlens_q, ctx.slot_of_seq, o, H, K, K,
-                        per_channel=True, w_bias=self.params["decay.bias"], bonus=self.params["bonus"])
+                        per_channel=True, w_bias=self.params["decay.bias"], bonus=self.params["bonus"],
+                        max_q_len=ctx.max_q_len)
         out = torch.empty((T, c), dtype=x.dtype, device=x.device)
         ops.group_norm_gate(o, H, self.params["norm.weight"], self.norm_eps, out, gate=g, gate_off=0, gate_first=False)
         return ops.linear(out, self.params["o.weight"], None, defer=True)

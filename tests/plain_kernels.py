@@ -342,7 +342,7 @@ class PlainKernels:
 
     def linear_scan(self, r, r_off, r_heads, k, k_off, k_heads, v, v_off, w, w_off, state, state_off, cu_seqlens_q,
                     slot_of_seq, out, heads, dim, vdim, per_channel=True, w_bias=None, v_scale=None, bonus=None,
-                    skip=None):
+                    skip=None, max_q_len=None):
         for b in range(slot_of_seq.numel()):
             lo, hi, slot = int(cu_seqlens_q[b]), int(cu_seqlens_q[b + 1]), int(slot_of_seq[b])
             if slot < 0:

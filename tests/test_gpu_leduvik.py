@@ -164,12 +164,12 @@ def test_step_sizes_and_decays():
 
 
 @pytest.mark.parametrize("H,K", [(5, 8), (2, 20), (6, 48), (2, 64), (1, 128), (3, 200)])
-@pytest.mark.parametrize("lens", [[37, 1, 5], [3, 70, 1]])
+@pytest.mark.parametrize("lens", [[37, 1, 5], [3, 70, 1], [200, 64, 129], [128, 1, 65]])
 def test_time_mix_recurrence_carries_its_state(H, K, lens):
     """The bonus recurrence over three requests in two steps against the plain token-by-token form; the state of a
     request travels in its slot, a padding request between them touches nothing."""
     ops = gpu_ops()
-    T2 = [9, 4, 20]
+    T2 = [9, 4, 20] if lens[0] < 100 else [1, 192, 70]      # beyond 64 tokens a request is worked in runs side by side
     bonus, bias = rnd((H, K), 1, 0.5), rnd((H * K,), 2) - 1.0
     state = torch.zeros((5, 7 + H * K * K), dtype=torch.float32, device=DEV)
     slots = [3, 0, 4]
@@ -203,7 +203,7 @@ def test_state_space_recurrence_carries_its_state(H, G, N, V):
     state = torch.zeros((3, 11 + H * N * V), dtype=torch.float32, device=DEV)
     slots = [2, 0]
     carried = [torch.zeros(H, N, V, dtype=torch.float64) for _ in slots]
-    for step, lens in enumerate([[45, 2], [1, 19], [70, 1]]):
+    for step, lens in enumerate([[45, 2], [1, 19], [70, 1], [256, 131], [64, 65]]):
         T = sum(lens)
         xbc = rnd((T, inner + 2 * G * N), 10 + step, 0.8)
         dt = pl.softplus(rnd((T, H), 20 + step).double())
