@@ -12,7 +12,7 @@
 // v may first be multiplied by a step size per (token, head), and o may receive skip[h] * (the unscaled v).  The
 // columns of S never meet, so a column lives in registers, spread over LPC adjacent lanes of 16 rows each.  A wave
 // owns 64 / LPC columns of one head; the waves of a block (up to four) own neighbouring columns and share what they
-// stage in LDS for 16 tokens at a time: r, k and the decays (formed on the way: as given, or exp(-exp(x + bias))),
+// stage in LDS for 16 (8 where a lane holds four columns) tokens at a time: r, k and the decays (formed on the way: as given, or exp(-exp(x + bias))),
 // the block's columns of v and the step sizes.
 //
 // Requests that bring no more than a run's length of tokens are walked by one block per (request, head, columns):
@@ -70,20 +70,40 @@ __device__ __forceinline__ bool scan_place(const ScanArgs& a, int b, int& seq, i
   return run >= 0 && run < runs;
 }
 
+// The sum of v over the LPC adjacent lanes that share a column, in each of them, by data-parallel permutes within a
+// row of 16 lanes (no trip through LDS): neighbours, pairs, then the mirrored half-row and row.
+template <int CTRL>
+__device__ __forceinline__ float scan_dpp_add(float v) {
+  return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+
+template <int LPC>
+__device__ __forceinline__ float scan_group_sum(float v) {
+  if constexpr (LPC >= 2) v = scan_dpp_add<0xB1>(v);    // quad_perm [1, 0, 3, 2]
+  if constexpr (LPC >= 4) v = scan_dpp_add<0x4E>(v);    // quad_perm [2, 3, 0, 1]
+  if constexpr (LPC >= 8) v = scan_dpp_add<0x141>(v);   // row_half_mirror
+  if constexpr (LPC >= 16) v = scan_dpp_add<0x140>(v);  // row_mirror
+  return v;
+}
+
 // PASS 0: a run with outputs (the whole request, or pass 3 of a long one); PASS 1: B and a of a run, no outputs.
-template <int PASS>
-__global__ void __launch_bounds__(64 * kScanWaves) linear_scan_kernel(ScanArgs a) {
-  extern __shared__ float staged[];          // [kScanStage][3 * KP + VW + 1, padded]: r, k, w, the block's v columns, step size
+// LPC lanes share a column's rows; a lane holds its 16 rows of CPL adjacent columns, so that a staged r, k or w
+// entry read from LDS serves CPL columns.
+template <int PASS, int LPC, int CPL, bool BEFORE>
+__global__ void __launch_bounds__(64 * kScanWaves) __attribute__((amdgpu_waves_per_eu(4)))
+linear_scan_kernel(ScanArgs a) {
+  constexpr int kStage = CPL > 1 ? kScanStage / 2 : kScanStage;   // wide lanes: half the LDS, so that more blocks fit
+  extern __shared__ float staged[];          // [kStage][3 * KP + VW + 1, padded]: r, k, w, the block's v columns, step size
   const int h = blockIdx.y;
-  const int lpc = a.lpc, cols = kWave / lpc;
-  const int KP = lpc * kScanRows;
-  const int VW = a.waves * cols;             // columns of v the block owns
+  constexpr int cols = kWave / LPC;          // lanes groups of a wave, CPL columns each
+  constexpr int KP = LPC * kScanRows;
+  const int VW = a.waves * cols * CPL;       // columns of v the block owns
   const int per_token = 3 * KP + ((VW + 4) & ~3);   // a token's rows stay 16-byte aligned
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int col0 = blockIdx.z * VW;
-  const int vcol = wave * cols + lane / lpc; // the lane's column among the block's
+  const int vcol = (wave * cols + lane / LPC) * CPL;   // the lane's first column among the block's
   const int col = col0 + vcol;
-  const int part = lane % lpc;               // which 16 rows of the column
+  const int part = lane % LPC;               // which 16 rows of the columns
   const int row0 = part * kScanRows;
   const int K = a.K, V = a.V;
   int seq, run, runs;
@@ -93,50 +113,68 @@ __global__ void __launch_bounds__(64 * kScanWaves) linear_scan_kernel(ScanArgs a
   const int t0 = a.run_len == 0 ? s0 : s0 + run * a.run_len;
   const int t1 = a.run_len == 0 ? s1 : min(s1, t0 + a.run_len);
   const int slot = a.slot_of_seq[seq];
-  const bool live = col < V;
   if (slot < 0) {                            // a padding row: nothing to carry, its output is never read
     if (PASS == 0)
       for (int t = t0; t < t1; ++t)
-        if (live && part == 0) a.out[(size_t)t * a.ldo + (size_t)h * V + col] = 0.f;
+        for (int c = 0; c < CPL; ++c)
+          if (col + c < V && part == 0) a.out[(size_t)t * a.ldo + (size_t)h * V + col + c] = 0.f;
     return;
   }
   const size_t place = a.run_len == 0 ? 0 : (size_t)(s0 / a.run_len + seq + run);
   float* S_slot = a.state + (size_t)slot * a.slot_stride + a.state_off + (size_t)h * K * V;
   float* S_run = a.run_state != nullptr ? a.run_state + (place * a.H + h) * (size_t)K * V : nullptr;
-  float S[kScanRows];
+  float S[CPL][kScanRows];
   if (PASS == 1) {
 #pragma unroll
-    for (int i = 0; i < kScanRows; ++i) S[i] = 0.f;
+    for (int c = 0; c < CPL; ++c)
+#pragma unroll
+      for (int i = 0; i < kScanRows; ++i) S[c][i] = 0.f;
   } else {
     const float* from = runs > 1 ? S_run : S_slot;
 #pragma unroll
-    for (int i = 0; i < kScanRows; ++i) S[i] = (live && row0 + i < K) ? from[(size_t)(row0 + i) * V + col] : 0.f;
+    for (int i = 0; i < kScanRows; ++i)
+#pragma unroll
+      for (int c = 0; c < CPL; ++c)
+        S[c][i] = (col + c < V && row0 + i < K) ? from[(size_t)(row0 + i) * V + col + c] : 0.f;
   }
   float u[kScanRows];                        // PASS 0: the bonus; PASS 1: the product of the run's decays
-  const bool before = a.bonus != nullptr;
+  constexpr bool before = BEFORE;
 #pragma unroll
   for (int i = 0; i < kScanRows; ++i)
     u[i] = PASS == 1 ? 1.f : ((before && row0 + i < K) ? a.bonus[(size_t)h * K + row0 + i] : 0.f);
   const float skip = a.skip != nullptr ? a.skip[h] : 0.f;
   const int rh = h / a.r_div, kh = h / a.k_div;
 
-  for (int base = t0; base < t1; base += kScanStage) {
-    const int n = min(kScanStage, t1 - base);
+  for (int base = t0; base < t1; base += kStage) {
+    const int n = min(kStage, t1 - base);
     __syncthreads();
-    for (int e = tid; e < n * KP; e += blockDim.x) {
-      const int j = e / KP, i = e - j * KP;
-      const size_t t = (size_t)(base + j);
-      float rv = 0.f, kv = 0.f, wv = 1.f;
-      if (i < K) {
-        if (PASS == 0) rv = a.r[t * a.ldr + (size_t)rh * K + i];
-        kv = a.k[t * a.ldk + (size_t)kh * K + i];
-        wv = a.w_per_channel ? a.w[t * a.ldw + (size_t)h * K + i] : a.w[t * a.ldw + h];
-        if (a.w_mode == 1) wv = expf(-expf(wv + a.w_bias[(size_t)h * K + i]));
+    // four entries a thread at a time, every load of the four asked for before the first is used
+    for (int e0 = tid; e0 < n * KP; e0 += 4 * blockDim.x) {
+      float rv[4], kv[4], wv[4], wb[4];
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        const int e = e0 + x * blockDim.x;
+        const int j = e / KP, i = e - j * KP;
+        const size_t t = (size_t)(base + j);
+        rv[x] = 0.f, kv[x] = 0.f, wv[x] = 1.f, wb[x] = 0.f;
+        if (e < n * KP && i < K) {
+          if (PASS == 0) rv[x] = a.r[t * a.ldr + (size_t)rh * K + i];
+          kv[x] = a.k[t * a.ldk + (size_t)kh * K + i];
+          wv[x] = a.w_per_channel ? a.w[t * a.ldw + (size_t)h * K + i] : a.w[t * a.ldw + h];
+          if (a.w_mode == 1) wb[x] = a.w_bias[(size_t)h * K + i];
+        }
       }
-      float* dst = staged + (size_t)j * per_token;
-      dst[i] = rv;
-      dst[KP + i] = kv;
-      dst[2 * KP + i] = wv;
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        const int e = e0 + x * blockDim.x;
+        if (e < n * KP) {
+          const int j = e / KP, i = e - j * KP;
+          float* dst = staged + (size_t)j * per_token;
+          dst[i] = rv[x];
+          dst[KP + i] = kv[x];
+          dst[2 * KP + i] = (a.w_mode == 1 && i < K) ? expf(-expf(wv[x] + wb[x])) : wv[x];
+        }
+      }
     }
     for (int e = tid; e < n * (VW + 1); e += blockDim.x) {
       const int j = e / (VW + 1), c = e - j * (VW + 1);
@@ -152,60 +190,78 @@ __global__ void __launch_bounds__(64 * kScanWaves) linear_scan_kernel(ScanArgs a
       const float4* r4 = reinterpret_cast<const float4*>(src + row0);
       const float4* k4 = reinterpret_cast<const float4*>(src + KP + row0);
       const float4* w4 = reinterpret_cast<const float4*>(src + 2 * KP + row0);
-      const float v_raw = src[3 * KP + vcol];
-      const float v = v_raw * src[3 * KP + VW];
-      float acc = 0.f;
+      const float step = src[3 * KP + VW];
+      float v_raw[CPL], v[CPL], acc[CPL];
+#pragma unroll
+      for (int c = 0; c < CPL; ++c) {
+        v_raw[c] = src[3 * KP + vcol + c];
+        v[c] = v_raw[c] * step;
+        acc[c] = 0.f;
+      }
 #pragma unroll
       for (int q = 0; q < kScanRows / 4; ++q) {
         const float4 kq = k4[q], wq = w4[q];
         const float kk[4] = {kq.x, kq.y, kq.z, kq.w}, ww[4] = {wq.x, wq.y, wq.z, wq.w};
         if (PASS == 1) {
 #pragma unroll
-          for (int c = 0; c < 4; ++c) {
-            S[4 * q + c] = ww[c] * S[4 * q + c] + kk[c] * v;
-            u[4 * q + c] *= ww[c];
+          for (int x = 0; x < 4; ++x) {
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) S[c][4 * q + x] = ww[x] * S[c][4 * q + x] + kk[x] * v[c];
+            u[4 * q + x] *= ww[x];
           }
         } else {
           const float4 rq = r4[q];
           const float rr[4] = {rq.x, rq.y, rq.z, rq.w};
           if (before) {
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-              const float kv = kk[c] * v;
-              acc += rr[c] * (S[4 * q + c] + u[4 * q + c] * kv);
-              S[4 * q + c] = ww[c] * S[4 * q + c] + kv;
+            for (int x = 0; x < 4; ++x) {
+              const float ru = rr[x] * u[4 * q + x];
+#pragma unroll
+              for (int c = 0; c < CPL; ++c) {
+                const float kv = kk[x] * v[c];
+                acc[c] += rr[x] * S[c][4 * q + x] + ru * kv;
+                S[c][4 * q + x] = ww[x] * S[c][4 * q + x] + kv;
+              }
             }
           } else {
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-              S[4 * q + c] = ww[c] * S[4 * q + c] + kk[c] * v;
-              acc += rr[c] * S[4 * q + c];
+            for (int x = 0; x < 4; ++x) {
+#pragma unroll
+              for (int c = 0; c < CPL; ++c) {
+                S[c][4 * q + x] = ww[x] * S[c][4 * q + x] + kk[x] * v[c];
+                acc[c] += rr[x] * S[c][4 * q + x];
+              }
             }
           }
         }
       }
       if (PASS == 0) {
-        for (int off = lpc >> 1; off > 0; off >>= 1) acc += __shfl_xor(acc, off, kWave);
-        if (live && part == 0) a.out[(size_t)(base + j) * a.ldo + (size_t)h * V + col] = acc + skip * v_raw;
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) {
+          const float sum = scan_group_sum<LPC>(acc[c]);
+          if (col + c < V && part == 0) a.out[(size_t)(base + j) * a.ldo + (size_t)h * V + col + c] = sum + skip * v_raw[c];
+        }
       }
     }
   }
   if (PASS == 1) {
-    if (live) {
 #pragma unroll
-      for (int i = 0; i < kScanRows; ++i)
-        if (row0 + i < K) S_run[(size_t)(row0 + i) * V + col] = S[i];
-    }
+    for (int i = 0; i < kScanRows; ++i)
+#pragma unroll
+      for (int c = 0; c < CPL; ++c)
+        if (col + c < V && row0 + i < K) S_run[(size_t)(row0 + i) * V + col + c] = S[c][i];
     if (col == 0) {
       float* decay = a.run_decay + (place * a.H + h) * (size_t)K;
 #pragma unroll
       for (int i = 0; i < kScanRows; ++i)
         if (row0 + i < K) decay[row0 + i] = u[i];
     }
-  } else if (live && run == runs - 1) {
+  } else if (run == runs - 1) {
 #pragma unroll
     for (int i = 0; i < kScanRows; ++i)
-      if (row0 + i < K) S_slot[(size_t)(row0 + i) * V + col] = S[i];
+#pragma unroll
+      for (int c = 0; c < CPL; ++c)
+        if (col + c < V && row0 + i < K) S_slot[(size_t)(row0 + i) * V + col + c] = S[c][i];
   }
 }
 
@@ -265,20 +321,39 @@ ATOM_EXPORT int atom_linear_scan(const float* r, long ldr, int r_div, const floa
   int lpc = 1;
   while (lpc * kScanRows < K) lpc <<= 1;
   const int cols = kWave / lpc;
-  const int waves = min(kScanWaves, (V + cols - 1) / cols);
-  const int vw = waves * cols;
+  // long requests in runs: four columns a lane, so that a staged row serves four columns, where that still leaves
+  // waves enough to fill the chip; otherwise one column a lane, which gives the most waves
+  const bool wide = run_len > 0 && V >= 4 * cols && need * H * ((V + 4 * cols - 1) / (4 * cols)) >= 2048;
+  const int cpl = wide ? 4 : 1;
+  const int waves = min(kScanWaves, (V + cols * cpl - 1) / (cols * cpl));
+  const int vw = waves * cols * cpl;
   const long blocks_x = run_len > 0 ? need : num_seqs;
   if (blocks_x > 0x7fffffff || H > 65535 || (V + vw - 1) / vw > 65535 || ((long)K * V + 255) / 256 > 65535) return ATOM_TOO_LARGE;
   ScanArgs a{r, ldr, r_div, k, ldk, k_div, v, ldv, w, ldw, w_per_channel, w_bias, w_mode, v_scale, ldvs, bonus, skip,
              out, ldo, state, slot_stride, state_off, cu_seqlens, slot_of_seq, num_seqs, H, K, V, lpc, waves, run_len,
              run_len > 0 ? run_state : nullptr, run_len > 0 ? run_decay : nullptr};
-  const size_t smem = (size_t)kScanStage * (3 * lpc * kScanRows + ((vw + 4) & ~3)) * sizeof(float);
+  const size_t smem = (size_t)(cpl > 1 ? kScanStage / 2 : kScanStage) * (3 * lpc * kScanRows + ((vw + 4) & ~3)) * sizeof(float);
   const dim3 grid((unsigned)blocks_x, H, (V + vw - 1) / vw), block(kWave * waves);
+#define ATOM_SCAN_LAUNCH(PASS, LPC, CPL)                                                                     \
+  if (PASS == 0 && bonus != nullptr)                                                                         \
+    hipLaunchKernelGGL((linear_scan_kernel<PASS, LPC, CPL, true>), grid, block, smem, stream, a);            \
+  else                                                                                                       \
+    hipLaunchKernelGGL((linear_scan_kernel<PASS, LPC, CPL, false>), grid, block, smem, stream, a)
+#define ATOM_SCAN_BY_LPC(PASS, CPL)                       \
+  switch (lpc) {                                          \
+    case 1: ATOM_SCAN_LAUNCH(PASS, 1, CPL); break;        \
+    case 2: ATOM_SCAN_LAUNCH(PASS, 2, CPL); break;        \
+    case 4: ATOM_SCAN_LAUNCH(PASS, 4, CPL); break;        \
+    case 8: ATOM_SCAN_LAUNCH(PASS, 8, CPL); break;        \
+    default: ATOM_SCAN_LAUNCH(PASS, 16, CPL); break;      \
+  }
   if (run_len > 0) {
-    hipLaunchKernelGGL(linear_scan_kernel<1>, grid, block, smem, stream, a);
+    if (cpl == 4) { ATOM_SCAN_BY_LPC(1, 4) } else { ATOM_SCAN_BY_LPC(1, 1) }
     hipLaunchKernelGGL(linear_scan_fold_kernel, dim3(num_seqs, H, (unsigned)(((long)K * V + 255) / 256)), dim3(256), 0, stream, a);
   }
-  hipLaunchKernelGGL(linear_scan_kernel<0>, grid, block, smem, stream, a);
+  if (cpl == 4) { ATOM_SCAN_BY_LPC(0, 4) } else { ATOM_SCAN_BY_LPC(0, 1) }
+#undef ATOM_SCAN_BY_LPC
+#undef ATOM_SCAN_LAUNCH
   return launch_status();
 }
 
