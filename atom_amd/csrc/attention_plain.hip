@@ -46,6 +46,7 @@ qkv_plain_write_kernel(const float* __restrict__ proj, long ld, T* __restrict__ 
   }
   if (slot >= 0) {
     const float* vr = row + (size_t)(H + G) * D;
+    #pragma unroll 4
     for (int e = threadIdx.x; e < G * DV; e += blockDim.x) {
       const int g = e / DV, i = e - g * DV;
       v_cache[(((size_t)page * G + g) * DP + i) * (size_t)page_size + off] = from_f32<T>(vr[e]);
@@ -105,6 +106,7 @@ mean_of_norms_kernel(NormedInputs in, int n, T* __restrict__ out, int width, flo
   for (int b = 0; b < n; ++b) {
     const T* row = (const T*)in.x[b] + t * width;
     float ss = 0.f;
+    #pragma unroll 4
     for (int i = threadIdx.x; i < width; i += blockDim.x) {
       const float v = to_f32(row[i]);
       ss += v * v;
@@ -112,10 +114,74 @@ mean_of_norms_kernel(NormedInputs in, int n, T* __restrict__ out, int width, flo
     inv[b] = 1.f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
   }
   const float share = 1.f / (float)n;
+  #pragma unroll 4
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     float sum = 0.f;
     for (int b = 0; b < n; ++b) sum += to_f32(((const T*)in.x[b])[t * width + i]) * inv[b] * in.w[b][i];
     out[t * width + i] = from_f32<T>(sum * share);
+  }
+}
+
+// Rows of up to 512 groups of 16 bytes: every input's row stays in registers, all loads asked for before the first is
+// used, one barrier pair for all the sums of squares.
+template <typename T>
+__global__ void __launch_bounds__(256)
+mean_of_norms_vec_kernel(NormedInputs in, int n, T* __restrict__ out, int width, float eps) {
+  constexpr int N = 16 / sizeof(T);
+  union Pack { uint4 raw; T e[N]; };
+  __shared__ float scratch[4][4];
+  const size_t t = blockIdx.x;
+  const int chunks = width / N;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  Pack x[4][2];
+#pragma unroll
+  for (int b = 0; b < 4; ++b)
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      const int c = threadIdx.x + r * 256;
+      x[b][r].raw = uint4{0u, 0u, 0u, 0u};
+      if (b < n && c < chunks) x[b][r].raw = reinterpret_cast<const uint4*>((const T*)in.x[b] + t * width)[c];
+    }
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    float ss = 0.f;
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+      for (int i = 0; i < N; ++i) ss += to_f32(x[b][r].e[i]) * to_f32(x[b][r].e[i]);
+    ss = wave_sum(ss);
+    if (lane == 0) scratch[b][wave] = ss;
+  }
+  __syncthreads();
+  float inv[4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b)
+    inv[b] = 1.f / sqrtf((scratch[b][0] + scratch[b][1] + scratch[b][2] + scratch[b][3]) / (float)width + eps);
+  const float share = 1.f / (float)n;
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    const int c = threadIdx.x + r * 256;
+    if (c < chunks) {
+      float sum[N];
+#pragma unroll
+      for (int i = 0; i < N; ++i) sum[i] = 0.f;
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+        if (b < n) {
+#pragma unroll
+          for (int q = 0; q < N / 4; ++q) {
+            const float4 w4 = *reinterpret_cast<const float4*>(in.w[b] + (size_t)c * N + 4 * q);
+            sum[4 * q] += to_f32(x[b][r].e[4 * q]) * inv[b] * w4.x;
+            sum[4 * q + 1] += to_f32(x[b][r].e[4 * q + 1]) * inv[b] * w4.y;
+            sum[4 * q + 2] += to_f32(x[b][r].e[4 * q + 2]) * inv[b] * w4.z;
+            sum[4 * q + 3] += to_f32(x[b][r].e[4 * q + 3]) * inv[b] * w4.w;
+          }
+        }
+      Pack res;
+#pragma unroll
+      for (int i = 0; i < N; ++i) res.e[i] = from_f32<T>(sum[i] * share);
+      reinterpret_cast<uint4*>(out + t * width)[c] = res.raw;
+    }
   }
 }
 
@@ -129,6 +195,14 @@ ATOM_EXPORT int atom_mean_of_norms(const void* const* xs, const float* const* ws
     in.w[b] = ws[b];
   }
   if (tokens == 0) return ATOM_OK;
+  const int per = dtype == ATOM_F32 ? 4 : 8;
+  bool vec = width % per == 0 && width / per <= 512 && (uintptr_t)out % 16 == 0;
+  for (int b = 0; b < n; ++b) vec = vec && ((uintptr_t)xs[b] | (uintptr_t)ws[b]) % 16 == 0;
+  if (vec) {
+    ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((mean_of_norms_vec_kernel<T>), dim3(tokens), dim3(256), 0, stream, in, n,
+                                                   (T*)out, width, eps));
+    return launch_status();
+  }
   ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((mean_of_norms_kernel<T>), dim3(tokens), dim3(256), 0, stream, in, n,
                                                  (T*)out, width, eps));
   return launch_status();
@@ -147,6 +221,7 @@ embedding_positions_kernel(const T* __restrict__ table, const T* __restrict__ ro
   p = p < 0 ? 0 : (p >= max_positions ? max_positions - 1 : p);
   const T* a = table + (size_t)id * width;
   const T* b = rows + (size_t)p * width;
+  #pragma unroll 4
   for (int i = threadIdx.x; i < width; i += blockDim.x) out[t * width + i] = to_f32(a[i]) + to_f32(b[i]);
 }
 
@@ -165,34 +240,52 @@ ATOM_EXPORT int atom_embedding_positions(const void* table, const void* rows, in
 // ------------------------------------------------------------------ an activation entry by entry
 
 // act 0: SiLU, 1: ReLU, 2: tanh-GELU, 3: the square of ReLU, 4: tanh
+__device__ __forceinline__ float unary_act_of(float z, int act) {
+  if (act == 0) return z / (1.f + expf(-z));
+  if (act == 1) return fmaxf(z, 0.f);
+  if (act == 2) return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  if (act == 3) {
+    const float p = fmaxf(z, 0.f);
+    return p * p;
+  }
+  return tanhf(z);
+}
+
 template <typename T>
 __global__ void unary_act_kernel(const T* __restrict__ x, T* __restrict__ out, int act, size_t total) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
-  const float z = to_f32(x[idx]);
-  float y;
-  if (act == 0) {
-    y = z / (1.f + expf(-z));
-  } else if (act == 1) {
-    y = fmaxf(z, 0.f);
-  } else if (act == 2) {
-    y = 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
-  } else if (act == 3) {
-    const float p = fmaxf(z, 0.f);
-    y = p * p;
-  } else {
-    y = tanhf(z);
-  }
-  out[idx] = from_f32<T>(y);
+  out[idx] = from_f32<T>(unary_act_of(to_f32(x[idx]), act));
+}
+
+// 16 bytes a thread: `groups` groups of 16 / sizeof(T) entries, both pointers 16-byte aligned
+template <typename T>
+__global__ void unary_act_vec_kernel(const T* __restrict__ x, T* __restrict__ out, int act, size_t groups) {
+  constexpr int N = 16 / sizeof(T);
+  const size_t g = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (g >= groups) return;
+  union Pack { uint4 raw; T e[N]; } in, res;
+  in.raw = reinterpret_cast<const uint4*>(x)[g];
+#pragma unroll
+  for (int i = 0; i < N; ++i) res.e[i] = from_f32<T>(unary_act_of(to_f32(in.e[i]), act));
+  reinterpret_cast<uint4*>(out)[g] = res.raw;
 }
 
 ATOM_EXPORT int atom_unary_act(const void* x, void* out, int dtype, long total, int act, hipStream_t stream) {
   if (total < 0 || act < 0 || act > 4 || x == nullptr || out == nullptr) return ATOM_BAD_SHAPE;
   if (total == 0) return ATOM_OK;
-  const size_t blocks = ((size_t)total + 255) / 256;
+  const int per = dtype == ATOM_F32 ? 4 : 8;
+  const bool vec = total % per == 0 && ((uintptr_t)x | (uintptr_t)out) % 16 == 0;
+  const size_t work = vec ? (size_t)total / per : (size_t)total;
+  const size_t blocks = (work + 255) / 256;
   if (blocks > 0x7fffffffu) return ATOM_TOO_LARGE;
-  ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((unary_act_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream,
-                                                 (const T*)x, (T*)out, act, (size_t)total));
+  if (vec) {
+    ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((unary_act_vec_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream,
+                                                   (const T*)x, (T*)out, act, work));
+  } else {
+    ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((unary_act_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream,
+                                                   (const T*)x, (T*)out, act, (size_t)total));
+  }
   return launch_status();
 }
 

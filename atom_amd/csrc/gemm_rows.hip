@@ -45,6 +45,7 @@ struct RowsParams {
   const float* g_next;   // residual: [n], the weight of the norm that follows
   int m, n, k, inter, out_f32, mode, ss_parts, kslice, per_wave, tiles;   // kslice: k of a slice; per_wave: slices a wave
   int cols;              // output columns of a block: 16, 12 or 8 (gate: 8 gate and 8 up rows)
+  int act;               // plain: an activation on the product (0 none, 1 SiLU, 2 ReLU, 3 tanh-GELU, 4 ReLU squared)
   float eps;
 };
 
@@ -236,6 +237,10 @@ __global__ void __launch_bounds__(512, (MR > 4 ? 3 : 4)) gemm_rows_kernel(RowsPa
     return;
   }
   if (has) {
+    if (p.act == 1) v = v / (1.f + expf(-v));
+    else if (p.act == 2) v = fmaxf(v, 0.f);
+    else if (p.act == 3) v = 0.5f * v * (1.f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+    else if (p.act == 4) v = fmaxf(v, 0.f) * fmaxf(v, 0.f);
     if (p.out_f32) reinterpret_cast<float*>(p.y)[(size_t)m * p.n + col] = v;
     else reinterpret_cast<bf16_t*>(p.y)[(size_t)m * p.n + col] = from_f32<bf16_t>(v);
   }
@@ -265,7 +270,8 @@ ATOM_EXPORT int atom_gemm_rows_supports(int m, int n, int k) {
   return m >= 1 && m <= 8 && n >= 1 && k >= 8 && k % 8 == 0;
 }
 
-// mode 0 (plain): y [m, n], bfloat16 or float32 (out_f32).   mode 1 (gate): w is [2 n, k], y [m, n] bfloat16.
+// mode 0 (plain): y [m, n], bfloat16 or float32 (out_f32), act(product + bias) with act 1 SiLU, 2 ReLU, 3 tanh-GELU,
+// 4 the square of ReLU (0: none).   mode 1 (gate): w is [2 n, k], y [m, n] bfloat16.
 // mode 2 (residual): res [m, n] float32 += product, ss_out [m, atom_gemm_rows_parts(n, cols)], and, with g_next [n],
 // xg_out [m, n] = bf16(res * g_next).
 // cols: output columns a block owns in modes 0 and 2: 16, or 12 or 8 for widths whose 16-column tiles would leave
@@ -276,8 +282,9 @@ ATOM_EXPORT int atom_gemm_rows_supports(int m, int n, int k) {
 ATOM_EXPORT int atom_gemm_rows(const void* x, const int* rows, const float* ss, int ss_parts, float eps, const void* w,
                                const float* bias, void* y, float* res, float* ss_out, void* xg_out,
                                const float* g_next, int m, int n, int k, int mode, int out_f32, int cols,
-                               int waves_override, hipStream_t stream) {
+                               int waves_override, int act, hipStream_t stream) {
   if (m < 0 || n <= 0 || k <= 0 || mode < 0 || mode > 2) return ATOM_BAD_SHAPE;
+  if (act < 0 || act > 4 || (act != 0 && mode != ROWS_PLAIN)) return ATOM_UNSUPPORTED;
   if (!rows_cols_ok(cols) || (mode == ROWS_GATE && cols != 16)) return ATOM_UNSUPPORTED;
   if (!atom_gemm_rows_supports(max(m, 1), n, k)) return ATOM_UNSUPPORTED;
   if (m == 0) return ATOM_OK;
@@ -293,6 +300,7 @@ ATOM_EXPORT int atom_gemm_rows(const void* x, const int* rows, const float* ss, 
   p.inter = mode == ROWS_GATE ? n : 0;
   p.tiles = rows_tiles(n, mode, cols);
   p.cols = cols;
+  p.act = act;
   int waves = rows_waves(m, p.tiles, k);
   if (waves_override == 4 || waves_override == 8) waves = waves_override;
   // 8 slices of K (4 where K is shorter than 8 quarters): the same for every number of rows and of waves

@@ -376,6 +376,7 @@ token_shift_kernel(const T* __restrict__ x, const float* __restrict__ mu, int n,
   const bool heads = t == first;             // the request's first token of this step
   const int last = padding ? t : cu_seqlens[seq + 1] - 1;
   float* kept = slot >= 0 ? state + (size_t)slot * slot_stride + state_off : nullptr;
+  #pragma unroll 4
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     const float cur = to_f32(row[i]);
     float prev;
@@ -391,6 +392,71 @@ token_shift_kernel(const T* __restrict__ x, const float* __restrict__ mu, int n,
   }
 }
 
+// The same with 16 bytes a thread and every load of a thread asked for before the first is used: widths that are a
+// multiple of 16 / sizeof(T), up to 8 mixes, rows and state rows 16-byte aligned.
+template <typename T>
+__global__ void __launch_bounds__(256)
+token_shift_vec_kernel(const T* __restrict__ x, const float* __restrict__ mu, int n, T* __restrict__ mixes,
+                       float* __restrict__ state, long slot_stride, long state_off, const int* __restrict__ cu_seqlens,
+                       const int* __restrict__ slot_of_seq, const int* __restrict__ token_seq, int tokens, int width) {
+  constexpr int N = 16 / sizeof(T);
+  union Pack { uint4 raw; T e[N]; };
+  const int t = blockIdx.x;
+  const int seq = token_seq[t];
+  const bool padding = seq < 0;
+  const int first = padding ? t : cu_seqlens[seq];
+  const int slot = padding ? -1 : slot_of_seq[seq];
+  const bool heads = t == first;
+  const int last = padding ? t : cu_seqlens[seq + 1] - 1;
+  float* kept = slot >= 0 ? state + (size_t)slot * slot_stride + state_off : nullptr;
+  for (int c = threadIdx.x; c < width / N; c += blockDim.x) {
+    const int i0 = c * N;
+    Pack cur, before, tail;
+    cur.raw = *reinterpret_cast<const uint4*>(x + (size_t)t * width + i0);
+    float prev[N];
+    if (heads) {
+      tail.raw = *reinterpret_cast<const uint4*>(x + (size_t)last * width + i0);
+#pragma unroll
+      for (int q = 0; q < N / 4; ++q) {
+        float4 k4 = kept != nullptr ? *reinterpret_cast<const float4*>(kept + i0 + 4 * q) : float4{0.f, 0.f, 0.f, 0.f};
+        prev[4 * q] = k4.x, prev[4 * q + 1] = k4.y, prev[4 * q + 2] = k4.z, prev[4 * q + 3] = k4.w;
+      }
+    } else {
+      before.raw = *reinterpret_cast<const uint4*>(x + (size_t)(t - 1) * width + i0);
+#pragma unroll
+      for (int i = 0; i < N; ++i) prev[i] = to_f32(before.e[i]);
+    }
+    float4 m[8][N / 4];
+#pragma unroll
+    for (int sx = 0; sx < 8; ++sx)
+      if (sx < n) {
+#pragma unroll
+        for (int q = 0; q < N / 4; ++q) m[sx][q] = *reinterpret_cast<const float4*>(mu + (size_t)sx * width + i0 + 4 * q);
+      }
+    if (heads && kept != nullptr) {
+#pragma unroll
+      for (int q = 0; q < N / 4; ++q)
+        *reinterpret_cast<float4*>(kept + i0 + 4 * q) = float4{to_f32(tail.e[4 * q]), to_f32(tail.e[4 * q + 1]),
+                                                                to_f32(tail.e[4 * q + 2]), to_f32(tail.e[4 * q + 3])};
+    }
+#pragma unroll
+    for (int sx = 0; sx < 8; ++sx)
+      if (sx < n) {
+        Pack res;
+#pragma unroll
+        for (int q = 0; q < N / 4; ++q) {
+          const float w4[4] = {m[sx][q].x, m[sx][q].y, m[sx][q].z, m[sx][q].w};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float cv = to_f32(cur.e[4 * q + i]);
+            res.e[4 * q + i] = from_f32<T>(cv + (prev[4 * q + i] - cv) * w4[i]);
+          }
+        }
+        *reinterpret_cast<uint4*>(mixes + ((size_t)sx * tokens + t) * width + i0) = res.raw;
+      }
+  }
+}
+
 ATOM_EXPORT int atom_token_shift(const void* x, int dtype, const float* mu, int n, void* mixes, float* state,
                                  long slot_stride, long state_off, const int* cu_seqlens, const int* slot_of_seq,
                                  const int* token_seq, int tokens, int width, hipStream_t stream) {
@@ -398,6 +464,15 @@ ATOM_EXPORT int atom_token_shift(const void* x, int dtype, const float* mu, int 
   if (x == nullptr || mu == nullptr || mixes == nullptr || state == nullptr) return ATOM_BAD_SHAPE;
   if (cu_seqlens == nullptr || slot_of_seq == nullptr || token_seq == nullptr) return ATOM_BAD_SHAPE;
   if (tokens == 0) return ATOM_OK;
+  const int per = dtype == ATOM_F32 ? 4 : 8;
+  const bool vec = n <= 8 && width % per == 0 && ((uintptr_t)x | (uintptr_t)mixes | (uintptr_t)mu | (uintptr_t)state) % 16 == 0 &&
+                   slot_stride % 4 == 0 && state_off % 4 == 0;
+  if (vec) {
+    ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((token_shift_vec_kernel<T>), dim3(tokens), dim3(256), 0, stream,
+                                                   (const T*)x, mu, n, (T*)mixes, state, slot_stride, state_off, cu_seqlens,
+                                                   slot_of_seq, token_seq, tokens, width));
+    return launch_status();
+  }
   ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((token_shift_kernel<T>), dim3(tokens), dim3(256), 0, stream, (const T*)x, mu,
                                                  n, (T*)mixes, state, slot_stride, state_off, cu_seqlens, slot_of_seq,
                                                  token_seq, tokens, width));
@@ -438,8 +513,8 @@ ATOM_EXPORT int atom_step_decay(const float* raw, long ld, const float* dt_bias,
 // out[t, g, :] = y / rms(y) * weight * silu(gate)      (gate_first 0: the gate multiplies the normed row)
 // out[t, g, :] = z / rms(z) * weight, z = y * silu(gate) (gate_first 1: the gate comes before the norm)
 // for each of `groups` equal parts of a row of y (float32); gate: float32 [T, ldg], the row's gate values from
-// column 0 (null: no gate); weight: float32 [groups * gw] (null: ones).  A block a token; a part no wider than 256 is summed
-// by one wave, a wider one by the whole block.
+// column 0 (null: no gate); weight: float32 [groups * gw] (null: ones).  A part no wider than 256 is summed by one wave (a row's parts spread
+// over the waves of up to 64 blocks), a wider one by the whole block of its token.
 __device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
 
 template <typename T>
@@ -454,7 +529,7 @@ group_norm_gate_kernel(const float* __restrict__ y, long ldy, const float* __res
   T* dst = out + t * (size_t)groups * gw;
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave, waves = blockDim.x / kWave;
   if (gw <= 256) {
-    for (int g = wave; g < groups; g += waves) {
+    for (int g = blockIdx.y * waves + wave; g < groups; g += gridDim.y * waves) {
       const int base = g * gw;
       float vals[4];
       float ss = 0.f;
@@ -486,12 +561,14 @@ group_norm_gate_kernel(const float* __restrict__ y, long ldy, const float* __res
   for (int g = 0; g < groups; ++g) {
     const int base = g * gw;
     float ss = 0.f;
+    #pragma unroll 4
     for (int i = threadIdx.x; i < gw; i += blockDim.x) {
       float v = yr[base + i];
       if (gate_first && gr != nullptr) v *= silu_f(gr[base + i]);
       ss += v * v;
     }
     const float inv = 1.f / sqrtf(block_sum(ss, scratch) / (float)gw + eps);
+    #pragma unroll 4
     for (int i = threadIdx.x; i < gw; i += blockDim.x) {
       float v = yr[base + i];
       const float s = gr != nullptr ? silu_f(gr[base + i]) : 1.f;
@@ -504,6 +581,55 @@ group_norm_gate_kernel(const float* __restrict__ y, long ldy, const float* __res
   }
 }
 
+// Parts wider than 256 entries whose rows are 16-byte aligned: a part's entries (up to 8,192) stay in registers, four
+// consecutive ones a load, every load asked for before the first is used; memory is read once.
+template <typename T>
+__global__ void __launch_bounds__(256)
+group_norm_gate_vec_kernel(const float* __restrict__ y, long ldy, const float* __restrict__ gate, long ldg,
+                           const float* __restrict__ weight, T* __restrict__ out, int groups, int gw, float eps,
+                           int gate_first) {
+  constexpr int PER = 8;
+  __shared__ float scratch[16];
+  const size_t t = blockIdx.x;
+  const float* yr = y + t * ldy;
+  const float* gr = gate != nullptr ? gate + t * ldg : nullptr;
+  T* dst = out + t * (size_t)groups * gw;
+  for (int g = 0; g < groups; ++g) {
+    const int base = g * gw;
+    float4 v[PER], sg[PER], w[PER];
+#pragma unroll
+    for (int r = 0; r < PER; ++r) {
+      const int i = (threadIdx.x + r * 256) * 4;
+      v[r] = sg[r] = float4{0.f, 0.f, 0.f, 0.f};
+      w[r] = float4{1.f, 1.f, 1.f, 1.f};
+      if (i < gw) {
+        v[r] = *reinterpret_cast<const float4*>(yr + base + i);
+        if (gr != nullptr) sg[r] = *reinterpret_cast<const float4*>(gr + base + i);
+        if (weight != nullptr) w[r] = *reinterpret_cast<const float4*>(weight + base + i);
+      }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int r = 0; r < PER; ++r) {
+      if (gr != nullptr) sg[r] = float4{silu_f(sg[r].x), silu_f(sg[r].y), silu_f(sg[r].z), silu_f(sg[r].w)};
+      else sg[r] = float4{1.f, 1.f, 1.f, 1.f};
+      if (gate_first) v[r] = float4{v[r].x * sg[r].x, v[r].y * sg[r].y, v[r].z * sg[r].z, v[r].w * sg[r].w};
+      ss += v[r].x * v[r].x + v[r].y * v[r].y + v[r].z * v[r].z + v[r].w * v[r].w;
+    }
+    const float inv = 1.f / sqrtf(block_sum(ss, scratch) / (float)gw + eps);
+#pragma unroll
+    for (int r = 0; r < PER; ++r) {
+      const int i = (threadIdx.x + r * 256) * 4;
+      if (i < gw) {
+        float o[4] = {v[r].x * inv * w[r].x, v[r].y * inv * w[r].y, v[r].z * inv * w[r].z, v[r].w * inv * w[r].w};
+        if (!gate_first) o[0] *= sg[r].x, o[1] *= sg[r].y, o[2] *= sg[r].z, o[3] *= sg[r].w;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) dst[base + i + x] = from_f32<T>(o[x]);
+      }
+    }
+  }
+}
+
 ATOM_EXPORT int atom_group_norm_gate(const float* y, long ldy, const float* gate, long ldg, const float* weight, void* out,
                                      int out_dtype, int tokens, int groups, int gw, float eps, int gate_first,
                                      hipStream_t stream) {
@@ -511,7 +637,16 @@ ATOM_EXPORT int atom_group_norm_gate(const float* y, long ldy, const float* gate
   if (gate != nullptr && ldg < (long)groups * gw) return ATOM_BAD_SHAPE;
   if (y == nullptr || out == nullptr) return ATOM_BAD_SHAPE;
   if (tokens == 0) return ATOM_OK;
-  ATOM_DISPATCH_DTYPE(out_dtype, hipLaunchKernelGGL((group_norm_gate_kernel<T>), dim3(tokens), dim3(256), 0, stream, y, ldy,
-                                                     gate, ldg, weight, (T*)out, groups, gw, eps, gate_first));
+  const bool vec = gw > 256 && gw <= 8192 && gw % 4 == 0 && ldy % 4 == 0 && (gate == nullptr || ldg % 4 == 0) &&
+                   ((uintptr_t)y | (uintptr_t)gate | (uintptr_t)weight) % 16 == 0;
+  if (vec) {
+    ATOM_DISPATCH_DTYPE(out_dtype, hipLaunchKernelGGL((group_norm_gate_vec_kernel<T>), dim3(tokens), dim3(256), 0, stream, y,
+                                                       ldy, gate, ldg, weight, (T*)out, groups, gw, eps, gate_first));
+    return launch_status();
+  }
+  // narrow parts: a wave a part, the parts of a row spread over blocks
+  const unsigned across = gw <= 256 ? (unsigned)min(64, (groups + 3) / 4) : 1u;
+  ATOM_DISPATCH_DTYPE(out_dtype, hipLaunchKernelGGL((group_norm_gate_kernel<T>), dim3(tokens, across), dim3(256), 0, stream, y,
+                                                     ldy, gate, ldg, weight, (T*)out, groups, gw, eps, gate_first));
   return launch_status();
 }

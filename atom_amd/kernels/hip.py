@@ -423,7 +423,7 @@ class HipKernels:
         return folded <= split
 
     def _rows_launch(self, x, weight, bias, mode: int, y=None, res=None, ss_out=None, xg_out=None, g_next=None,
-                     out_f32: bool = False):
+                     out_f32: bool = False, act: int = 0):
         m, k = x.shape
         n = weight.shape[0] // 2 if mode == 1 else weight.shape[0]
         self._check("linear weight", weight, torch.bfloat16, (weight.shape[0], k))
@@ -440,7 +440,7 @@ class HipKernels:
             head = (_ptr(x), None, None, 0, ctypes.c_float(0.0))
         self._done("gemm_rows", self.lib.atom_gemm_rows(
             *head, _ptr(weight), _ptr(bias), _ptr(y), _ptr(res), _ptr(ss_out), _ptr(xg_out), _ptr(g_next), m, n, k,
-            mode, int(out_f32), 16 if mode == 1 else self.rows_cols(n), int(self.rows_waves), self._stream()))
+            mode, int(out_f32), 16 if mode == 1 else self.rows_cols(n), int(self.rows_waves), act, self._stream()))
 
     def _rows_product(self, x, weight, bias, out_dtype):
         y = torch.empty((x.shape[0], weight.shape[0]), dtype=out_dtype, device=weight.device)
@@ -824,6 +824,24 @@ class HipKernels:
             _ptr(x), self._code(x), _ptr(weight), self._code(weight), _ptr(bias), _ptr(y), self._code(y), m, n, k,
             self._stream()))
         return y
+
+    _ROWS_ACT = {"silu": 1, "relu": 2, "gelu_tanh": 3, "relu_squared": 4}
+
+    def linear_act(self, x, weight, bias, activation: str):
+        """``act(x @ weight.T + bias)`` in ``x``'s type: one kernel where the few-rows product takes it (a pending
+        norm of ``x`` folded in as well), else the product and the activation entry by entry."""
+        if activation not in self._ROWS_ACT:
+            raise KernelError(f"linear_act: unknown activation {activation!r}; known: {sorted(self._ROWS_ACT)}")
+        if isinstance(x, (DeferredSum, PendingProduct)):
+            x = self.materialize(x)
+        m = x.shape[0]
+        if m and self._rows_takes(x, weight):
+            y = torch.empty((m, weight.shape[0]), dtype=x.dtype, device=weight.device)
+            self._rows_launch(x, weight, bias, 0, y=y, act=self._ROWS_ACT[activation])
+            return y
+        up = self.linear(x, weight, bias)
+        out = torch.empty(tuple(up.shape), dtype=up.dtype, device=up.device)
+        return self.unary_act(up, out, activation)
 
     def linear_silu(self, x, weight, bias=None):
         """``silu(x @ Wg.T + bg) * (x @ Wu.T + bu)`` for ``weight`` = gate rows then up rows: one kernel

@@ -53,7 +53,7 @@ class GatedMLP(FeedForward):
 
 class DenseMLP(FeedForward):
     """``down(act(up(x)))`` without a gate; ``activation`` one of silu, relu, gelu_tanh, relu_squared (the square
-    of ReLU).  The activation is one elementwise kernel on the up product."""
+    of ReLU).  The activation is the up product's epilogue where its kernel offers one, else an elementwise kernel."""
 
     accepts_deferred = True   # the input goes to the up product as it is
 
@@ -75,9 +75,7 @@ class DenseMLP(FeedForward):
 
     def forward(self, ctx, x):
         ops = ctx.ops
-        up = ops.linear(x, self.params["up.weight"], None)
-        act = torch.empty(tuple(up.shape), dtype=up.dtype, device=up.device)
-        ops.unary_act(up, act, self.activation)
+        act = ops.linear_act(x, self.params["up.weight"], None, self.activation)
         return ops.linear(act, self.params["down.weight"], None, defer=True)
 
 

@@ -20,7 +20,7 @@ import zlib
 import torch
 
 # inner size of the decay's two products in a time-mixing branch: a tensor's shape says it, the configuration does not
-RANKS = {"A": 3, "B": 7, "C": 16, "X": 24}
+RANKS = {"A": 3, "B": 7, "C": 16, "D": 5, "X": 24}
 
 
 def _ssm(heads, vdim, state, groups, conv, norm_groups):
@@ -91,8 +91,21 @@ LEDU_X = {
     ],
 }
 
-CONFIGS = {"A": LEDU_A, "B": LEDU_B, "C": LEDU_C, "X": LEDU_X}
-SEEDS = {"A": 7, "B": 17, "C": 29, "X": 41}
+# D: odd sizes throughout (a width that is no multiple of 8, heads of 7, 9 and 11 entries, as many groups as heads in
+# the state-space mixer), attention first, the loop over the last two layers
+LEDU_D = {
+    "architecture": "Leduvik", "vocab": 77, "width": 52, "max_positions": 300, "norm": {"eps": 1e-5},
+    "logit_scale": 1.3, "loop": {"start": 1, "stop": 3, "times": 2},
+    "layers": [
+        {"type": "attention", "mixer": _attn(5, 5, 7, 9, 0.4, window=11), "mlp": _dense(30)},
+        {"type": "mamba2", "mixer": _ssm(3, 7, 9, 3, 3, 1), "mlp": _dense(34)},
+        {"type": "parallel", "mixer": {"left": _attn(3, 1, 9, 5, 0.3, temp=(0.4, 5)), "right": {"heads": 3, "dim": 11}},
+         "mlp": None},
+    ],
+}
+
+CONFIGS = {"A": LEDU_A, "B": LEDU_B, "C": LEDU_C, "D": LEDU_D, "X": LEDU_X}
+SEEDS = {"A": 7, "B": 17, "C": 29, "D": 5, "X": 41}
 
 
 def _draw(name: str, shape, seed: int) -> torch.Tensor:

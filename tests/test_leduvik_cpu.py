@@ -18,7 +18,7 @@ from atom_amd.config.model_config import LeduvikConfig
 from atom_amd.engine.core import StepEntry, load_model
 from atom_amd.weights.loader import expected_tensors
 
-LENGTHS = {"A": [1, 7, 33, 70], "B": [2, 19, 45, 64], "C": [3, 52]}
+LENGTHS = {"A": [1, 7, 33, 70], "B": [2, 19, 45, 64], "C": [3, 52], "D": [1, 30, 66]}
 
 
 def _requests(which, seed=0):
@@ -130,7 +130,7 @@ def test_config_reads_every_size_and_round_trips():
     assert build_model(model_config_from_dict(once)).join is None
 
 
-@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
 def test_names_and_shapes_are_the_designs(which):
     """The engine's list of checkpoint tensors, once the checkpoint's shapes have said the inner size of the decay's
     two products, is the design's list."""
@@ -170,7 +170,7 @@ def test_config_refuses_what_does_not_fit(path, value):
 # ------------------------------------------------------------------ the engine's bookkeeping
 
 
-@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("cut", ["whole", "tail", "portions", "mixed"])
 def test_cuts_match_plain(which, cut):
     requests = _requests(which)
