@@ -45,7 +45,7 @@ struct RowsParams {
   const float* g_next;   // residual: [n], the weight of the norm that follows
   int m, n, k, inter, out_f32, mode, ss_parts, kslice, per_wave, tiles;   // kslice: k of a slice; per_wave: slices a wave
   int cols;              // output columns of a block: 16, 12 or 8 (gate: 8 gate and 8 up rows)
-  int act;               // plain: an activation on the product (0 none, 1 SiLU, 2 ReLU, 3 tanh-GELU, 4 ReLU squared)
+  int act;               // plain: an activation on the product (0 none, 1 SiLU, 2 ReLU, 3 tanh-GELU, 4 ReLU squared, 5 tanh)
   float eps;
 };
 
@@ -241,6 +241,7 @@ __global__ void __launch_bounds__(512, (MR > 4 ? 3 : 4)) gemm_rows_kernel(RowsPa
     else if (p.act == 2) v = fmaxf(v, 0.f);
     else if (p.act == 3) v = 0.5f * v * (1.f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
     else if (p.act == 4) v = fmaxf(v, 0.f) * fmaxf(v, 0.f);
+    else if (p.act == 5) v = tanhf(v);
     if (p.out_f32) reinterpret_cast<float*>(p.y)[(size_t)m * p.n + col] = v;
     else reinterpret_cast<bf16_t*>(p.y)[(size_t)m * p.n + col] = from_f32<bf16_t>(v);
   }
@@ -271,7 +272,7 @@ ATOM_EXPORT int atom_gemm_rows_supports(int m, int n, int k) {
 }
 
 // mode 0 (plain): y [m, n], bfloat16 or float32 (out_f32), act(product + bias) with act 1 SiLU, 2 ReLU, 3 tanh-GELU,
-// 4 the square of ReLU (0: none).   mode 1 (gate): w is [2 n, k], y [m, n] bfloat16.
+// 4 the square of ReLU, 5 tanh (0: none).   mode 1 (gate): w is [2 n, k], y [m, n] bfloat16.
 // mode 2 (residual): res [m, n] float32 += product, ss_out [m, atom_gemm_rows_parts(n, cols)], and, with g_next [n],
 // xg_out [m, n] = bf16(res * g_next).
 // cols: output columns a block owns in modes 0 and 2: 16, or 12 or 8 for widths whose 16-column tiles would leave
@@ -284,7 +285,7 @@ ATOM_EXPORT int atom_gemm_rows(const void* x, const int* rows, const float* ss, 
                                const float* g_next, int m, int n, int k, int mode, int out_f32, int cols,
                                int waves_override, int act, hipStream_t stream) {
   if (m < 0 || n <= 0 || k <= 0 || mode < 0 || mode > 2) return ATOM_BAD_SHAPE;
-  if (act < 0 || act > 4 || (act != 0 && mode != ROWS_PLAIN)) return ATOM_UNSUPPORTED;
+  if (act < 0 || act > 5 || (act != 0 && mode != ROWS_PLAIN)) return ATOM_UNSUPPORTED;
   if (!rows_cols_ok(cols) || (mode == ROWS_GATE && cols != 16)) return ATOM_UNSUPPORTED;
   if (!atom_gemm_rows_supports(max(m, 1), n, k)) return ATOM_UNSUPPORTED;
   if (m == 0) return ATOM_OK;

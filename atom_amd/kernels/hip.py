@@ -825,10 +825,10 @@ class HipKernels:
             self._stream()))
         return y
 
-    _ROWS_ACT = {"silu": 1, "relu": 2, "gelu_tanh": 3, "relu_squared": 4}
+    _ROWS_ACT = {"silu": 1, "relu": 2, "gelu_tanh": 3, "relu_squared": 4, "tanh": 5}
 
-    def linear_act(self, x, weight, bias, activation: str):
-        """``act(x @ weight.T + bias)`` in ``x``'s type: one kernel where the few-rows product takes it (a pending
+    def linear_act(self, x, weight, bias, activation: str, out_dtype=None):
+        """``act(x @ weight.T + bias)`` in ``x``'s type (or ``out_dtype``): one kernel where the few-rows product takes it (a pending
         norm of ``x`` folded in as well), else the product and the activation entry by entry."""
         if activation not in self._ROWS_ACT:
             raise KernelError(f"linear_act: unknown activation {activation!r}; known: {sorted(self._ROWS_ACT)}")
@@ -836,10 +836,10 @@ class HipKernels:
             x = self.materialize(x)
         m = x.shape[0]
         if m and self._rows_takes(x, weight):
-            y = torch.empty((m, weight.shape[0]), dtype=x.dtype, device=weight.device)
-            self._rows_launch(x, weight, bias, 0, y=y, act=self._ROWS_ACT[activation])
+            y = torch.empty((m, weight.shape[0]), dtype=out_dtype or x.dtype, device=weight.device)
+            self._rows_launch(x, weight, bias, 0, y=y, act=self._ROWS_ACT[activation], out_f32=y.dtype == torch.float32)
             return y
-        up = self.linear(x, weight, bias)
+        up = self.linear(x, weight, bias, out_dtype=out_dtype)
         out = torch.empty(tuple(up.shape), dtype=up.dtype, device=up.device)
         return self.unary_act(up, out, activation)
 

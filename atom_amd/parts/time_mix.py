@@ -78,9 +78,7 @@ class TimeMixRecurrence(Mixer):
         # each of r, k, v and the gate reads a mix of its own
         r, k, v, g = (ops.linear(mixes[i], self.params[f"{name}.weight"], None, out_dtype=torch.float32)
                       for i, name in enumerate(("r", "k", "v", "gate")))
-        low = ops.linear(mixes[4], self.params["decay1.weight"], None, out_dtype=torch.float32)
-        squashed = torch.empty((T, rank), dtype=torch.float32, device=x.device)
-        ops.unary_act(low, squashed, "tanh")
+        squashed = ops.linear_act(mixes[4], self.params["decay1.weight"], None, "tanh", out_dtype=torch.float32)
         raw = torch.empty((T, c), dtype=torch.float32, device=x.device)
         ops.heads_gemm(squashed, 0, rank, 0, self.params["decay2.weight"].view(1, c, rank), raw, 0, c, 0, 1, T, c, rank,
                        exact=True)

@@ -114,9 +114,9 @@ class PlainKernels:
             y = y + bias.to(WIDE)
         return y.to(out_dtype or x.dtype)
 
-    def linear_act(self, x, weight, bias, activation):
+    def linear_act(self, x, weight, bias, activation, out_dtype=None):
         up = self.linear(x, weight, bias, out_dtype=WIDE)
-        return self.unary_act(up, torch.empty(tuple(up.shape), dtype=x.dtype), activation)
+        return self.unary_act(up, torch.empty(tuple(up.shape), dtype=out_dtype or x.dtype), activation)
 
     def linear_silu(self, x, weight, bias=None):
         return silu_and_mul(self.linear(x, weight, bias, out_dtype=WIDE)).to(x.dtype)

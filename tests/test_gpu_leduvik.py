@@ -93,6 +93,9 @@ def test_product_with_its_activation(dtype, rows):
         got = ops.linear_act(x.to(DEV), w.to(DEV), None, name)
         assert got.dtype == dtype and tuple(got.shape) == (rows, n)
         close(got, fn(x.double() @ w.double().T), dtype, f"{name}, {rows} rows")
+    wide = ops.linear_act(x.to(DEV), w.to(DEV), None, "tanh", out_dtype=torch.float32)
+    assert wide.dtype == torch.float32
+    close(wide, torch.tanh(x.double() @ w.double().T), dtype, f"tanh in float32, {rows} rows")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
