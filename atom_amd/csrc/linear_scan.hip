@@ -90,7 +90,9 @@ __device__ __forceinline__ float scan_group_sum(float v) {
 // LPC lanes share a column's rows; a lane holds its 16 rows of CPL adjacent columns, so that a staged r, k or w
 // entry read from LDS serves CPL columns.
 template <int PASS, int LPC, int CPL, bool BEFORE>
-__global__ void __launch_bounds__(64 * kScanWaves) __attribute__((amdgpu_waves_per_eu(4)))
+// (four waves a SIMD, 128 registers; the walk with a bonus and four columns a lane needs more and takes two)
+__global__ void __launch_bounds__(64 * kScanWaves)
+__attribute__((amdgpu_waves_per_eu(PASS == 0 && BEFORE && CPL > 1 ? 2 : 4)))
 linear_scan_kernel(ScanArgs a) {
   constexpr int kStage = CPL > 1 ? kScanStage / 2 : kScanStage;   // wide lanes: half the LDS, so that more blocks fit
   extern __shared__ float staged[];          // [kStage][3 * KP + VW + 1, padded]: r, k, w, the block's v columns, step size
