@@ -1,6 +1,7 @@
 // y[M, N] = x[M, K] * w[N, K]^T (+ bias[N]) in true float32: plain FMA, no matrix
-// cores, no reduced-precision mode.  Each output element is one sum over k in
-// ascending order, whatever M is, so a row's result does not depend on its batch.
+// cores, no reduced-precision mode.  Each output element is a sum over k in ascending
+// order, 16 terms at a time summed apart and then added to the long sum, whatever M
+// is, so a row's result does not depend on its batch.
 //
 // 64 x 64 tiles, 256 threads, each thread a 4 x 4 patch; K is walked 16 at a time
 // through LDS.  Any M, N, K (edges are guarded).
@@ -35,6 +36,7 @@ gemm_f32_kernel(const TX* __restrict__ x, const TW* __restrict__ w, const float*
       ws[lk + i][lrow] = (wr < n && kk < k) ? to_f32(w[(size_t)wr * k + kk]) : 0.f;
     }
     __syncthreads();
+    float part[4][4] = {};   // the step's 16 terms are summed apart and join the long sum as one: shorter chains, less rounding
 #pragma unroll
     for (int kk = 0; kk < kStep; ++kk) {
       float a[4], b[4];
@@ -45,8 +47,12 @@ gemm_f32_kernel(const TX* __restrict__ x, const TW* __restrict__ w, const float*
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        for (int j = 0; j < 4; ++j) part[i][j] = fmaf(a[i], b[j], part[i][j]);
     }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] += part[i][j];
     __syncthreads();
   }
 #pragma unroll
