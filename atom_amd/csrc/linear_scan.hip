@@ -39,7 +39,9 @@ struct ScanArgs {
   const float* k; long ldk; int k_div;
   const float* v; long ldv;                  // [T, H * V] at v
   const float* w; long ldw; int w_per_channel;   // [T, H * K] or [T, H]
-  const float* w_bias; int w_mode;           // 0: w is the decay; 1: decay = exp(-exp(w + w_bias[h * K + i]))
+  const float* w_bias; int w_mode;           // 0: w is the decay; 1: decay = exp(-exp(w + w_bias[h * K + i]));
+                                             // 2 (one decay per head): step = softplus(w + w_bias[h]) multiplies v,
+  const float* a_log;                        //    decay = exp(-exp(a_log[h]) step)
   const float* v_scale; long ldvs;           // [T, H] or null
   const float* bonus;                        // [H, K]: read_before; null: read_after
   const float* skip;                         // [H] or null
@@ -89,18 +91,20 @@ __device__ __forceinline__ float scan_group_sum(float v) {
 // PASS 0: a run with outputs (the whole request, or pass 3 of a long one); PASS 1: B and a of a run, no outputs.
 // LPC lanes share a column's rows; a lane holds its 16 rows of CPL adjacent columns, so that a staged r, k or w
 // entry read from LDS serves CPL columns.
-template <int PASS, int LPC, int CPL, bool BEFORE>
+// PERHEAD: one decay per head, staged once per token instead of once per row.
+template <int PASS, int LPC, int CPL, bool BEFORE, bool PERHEAD>
 // (four waves a SIMD, 128 registers; the walk with a bonus and four columns a lane needs more and takes two)
 __global__ void __launch_bounds__(64 * kScanWaves)
 __attribute__((amdgpu_waves_per_eu(PASS == 0 && BEFORE && CPL > 1 ? 2 : 4)))
 linear_scan_kernel(ScanArgs a) {
   constexpr int kStage = CPL > 1 ? kScanStage / 2 : kScanStage;   // wide lanes: half the LDS, so that more blocks fit
-  extern __shared__ float staged[];          // [kStage][3 * KP + VW + 1, padded]: r, k, w, the block's v columns, step size
+  extern __shared__ float staged[];          // [kStage][NW * KP + VW + 2, padded]: r, k, (w), the block's v columns, step, decay
   const int h = blockIdx.y;
   constexpr int cols = kWave / LPC;          // lanes groups of a wave, CPL columns each
   constexpr int KP = LPC * kScanRows;
   const int VW = a.waves * cols * CPL;       // columns of v the block owns
-  const int per_token = 3 * KP + ((VW + 4) & ~3);   // a token's rows stay 16-byte aligned
+  constexpr int NW = PERHEAD ? 2 : 3;        // rows of K entries staged per token
+  const int per_token = NW * KP + ((VW + 5) & ~3);   // a token's rows stay 16-byte aligned
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int col0 = blockIdx.z * VW;
   const int vcol = (wave * cols + lane / LPC) * CPL;   // the lane's first column among the block's
@@ -162,8 +166,10 @@ linear_scan_kernel(ScanArgs a) {
         if (e < n * KP && i < K) {
           if (PASS == 0) rv[x] = a.r[t * a.ldr + (size_t)rh * K + i];
           kv[x] = a.k[t * a.ldk + (size_t)kh * K + i];
-          wv[x] = a.w_per_channel ? a.w[t * a.ldw + (size_t)h * K + i] : a.w[t * a.ldw + h];
-          if (a.w_mode == 1) wb[x] = a.w_bias[(size_t)h * K + i];
+          if (!PERHEAD) {
+            wv[x] = a.w_per_channel ? a.w[t * a.ldw + (size_t)h * K + i] : a.w[t * a.ldw + h];
+            if (a.w_mode == 1) wb[x] = a.w_bias[(size_t)h * K + i];
+          }
         }
       }
 #pragma unroll
@@ -174,35 +180,50 @@ linear_scan_kernel(ScanArgs a) {
           float* dst = staged + (size_t)j * per_token;
           dst[i] = rv[x];
           dst[KP + i] = kv[x];
-          dst[2 * KP + i] = (a.w_mode == 1 && i < K) ? expf(-expf(wv[x] + wb[x])) : wv[x];
+          if (!PERHEAD) dst[2 * KP + i] = (a.w_mode == 1 && i < K) ? expf(-expf(wv[x] + wb[x])) : wv[x];
         }
       }
     }
-    for (int e = tid; e < n * (VW + 1); e += blockDim.x) {
-      const int j = e / (VW + 1), c = e - j * (VW + 1);
+    for (int e = tid; e < n * (VW + 2); e += blockDim.x) {
+      const int j = e / (VW + 2), c = e - j * (VW + 2);
       const size_t t = (size_t)(base + j);
       float x;
-      if (c == VW) x = a.v_scale != nullptr ? a.v_scale[t * a.ldvs + h] : 1.f;
-      else x = col0 + c < V ? a.v[t * a.ldv + (size_t)h * V + col0 + c] : 0.f;
-      staged[(size_t)j * per_token + 3 * KP + c] = x;
+      if (c >= VW) {                           // the token's step size, then (one decay per head) its decay
+        float step = a.v_scale != nullptr ? a.v_scale[t * a.ldvs + h] : 1.f;
+        float decay = 1.f;
+        if (PERHEAD) {
+          decay = a.w[t * a.ldw + h];
+          if (a.w_mode == 2) {
+            const float z = decay + a.w_bias[h];
+            step = z > 20.f ? z : log1pf(expf(z));
+            decay = expf(-expf(a.a_log[h]) * step);
+          }
+        }
+        x = c == VW ? step : decay;
+      } else {
+        x = col0 + c < V ? a.v[t * a.ldv + (size_t)h * V + col0 + c] : 0.f;
+      }
+      staged[(size_t)j * per_token + NW * KP + c] = x;
     }
     __syncthreads();
     for (int j = 0; j < n; ++j) {
       const float* src = staged + (size_t)j * per_token;
       const float4* r4 = reinterpret_cast<const float4*>(src + row0);
       const float4* k4 = reinterpret_cast<const float4*>(src + KP + row0);
-      const float4* w4 = reinterpret_cast<const float4*>(src + 2 * KP + row0);
-      const float step = src[3 * KP + VW];
+      const float4* w4 = reinterpret_cast<const float4*>(src + (NW - 1) * KP + row0);   // PERHEAD: not read
+      const float step = src[NW * KP + VW];
+      const float head_decay = src[NW * KP + VW + 1];
       float v_raw[CPL], v[CPL], acc[CPL];
 #pragma unroll
       for (int c = 0; c < CPL; ++c) {
-        v_raw[c] = src[3 * KP + vcol + c];
+        v_raw[c] = src[NW * KP + vcol + c];
         v[c] = v_raw[c] * step;
         acc[c] = 0.f;
       }
 #pragma unroll
       for (int q = 0; q < kScanRows / 4; ++q) {
-        const float4 kq = k4[q], wq = w4[q];
+        const float4 kq = k4[q];
+        const float4 wq = PERHEAD ? float4{head_decay, head_decay, head_decay, head_decay} : w4[q];
         const float kk[4] = {kq.x, kq.y, kq.z, kq.w}, ww[4] = {wq.x, wq.y, wq.z, wq.w};
         if (PASS == 1) {
 #pragma unroll
@@ -305,15 +326,17 @@ __global__ void __launch_bounds__(256) linear_scan_fold_kernel(ScanArgs a) {
 
 ATOM_EXPORT int atom_linear_scan(const float* r, long ldr, int r_div, const float* k, long ldk, int k_div, const float* v,
                                  long ldv, const float* w, long ldw, int w_per_channel, const float* w_bias, int w_mode,
-                                 const float* v_scale, long ldvs, const float* bonus, const float* skip, float* out,
+                                 const float* a_log, const float* v_scale, long ldvs, const float* bonus, const float* skip, float* out,
                                  long ldo, float* state, long slot_stride, long state_off, const int* cu_seqlens,
                                  const int* slot_of_seq, int num_seqs, int H, int K, int V, int tokens, int run_len,
                                  float* run_state, float* run_decay, long places, hipStream_t stream) {
   if (H <= 0 || K <= 0 || V <= 0 || num_seqs < 0 || r_div <= 0 || k_div <= 0 || tokens < 0) return ATOM_BAD_SHAPE;
   if (r == nullptr || k == nullptr || v == nullptr || w == nullptr || out == nullptr || state == nullptr) return ATOM_BAD_SHAPE;
   if (cu_seqlens == nullptr || slot_of_seq == nullptr) return ATOM_BAD_SHAPE;
-  if (w_mode != 0 && w_mode != 1) return ATOM_UNSUPPORTED;
+  if (w_mode < 0 || w_mode > 2) return ATOM_UNSUPPORTED;
   if (w_mode == 1 && (w_bias == nullptr || !w_per_channel)) return ATOM_BAD_SHAPE;
+  if (w_mode == 2 && (w_bias == nullptr || a_log == nullptr || w_per_channel)) return ATOM_BAD_SHAPE;
+  if (w_mode == 2 && (bonus != nullptr || v_scale != nullptr)) return ATOM_UNSUPPORTED;
   if (state_off < 0 || slot_stride < state_off + (long)H * K * V) return ATOM_BAD_SHAPE;
   if (K > 16 * kScanRows) return ATOM_TOO_LARGE;
   if (run_len < 0 || run_len % kScanStage) return ATOM_BAD_SHAPE;
@@ -331,16 +354,20 @@ ATOM_EXPORT int atom_linear_scan(const float* r, long ldr, int r_div, const floa
   const int vw = waves * cols * cpl;
   const long blocks_x = run_len > 0 ? need : num_seqs;
   if (blocks_x > 0x7fffffff || H > 65535 || (V + vw - 1) / vw > 65535 || ((long)K * V + 255) / 256 > 65535) return ATOM_TOO_LARGE;
-  ScanArgs a{r, ldr, r_div, k, ldk, k_div, v, ldv, w, ldw, w_per_channel, w_bias, w_mode, v_scale, ldvs, bonus, skip,
+  ScanArgs a{r, ldr, r_div, k, ldk, k_div, v, ldv, w, ldw, w_per_channel, w_bias, w_mode, a_log, v_scale, ldvs, bonus, skip,
              out, ldo, state, slot_stride, state_off, cu_seqlens, slot_of_seq, num_seqs, H, K, V, lpc, waves, run_len,
              run_len > 0 ? run_state : nullptr, run_len > 0 ? run_decay : nullptr};
-  const size_t smem = (size_t)(cpl > 1 ? kScanStage / 2 : kScanStage) * (3 * lpc * kScanRows + ((vw + 4) & ~3)) * sizeof(float);
+  const bool perhead = !w_per_channel && bonus == nullptr;   // one staged decay a token instead of one a row
+  const size_t smem = (size_t)(cpl > 1 ? kScanStage / 2 : kScanStage) *
+                      ((perhead ? 2 : 3) * lpc * kScanRows + ((vw + 5) & ~3)) * sizeof(float);
   const dim3 grid((unsigned)blocks_x, H, (V + vw - 1) / vw), block(kWave * waves);
 #define ATOM_SCAN_LAUNCH(PASS, LPC, CPL)                                                                     \
-  if (PASS == 0 && bonus != nullptr)                                                                         \
-    hipLaunchKernelGGL((linear_scan_kernel<PASS, LPC, CPL, true>), grid, block, smem, stream, a);            \
+  if (perhead)                                                                                               \
+    hipLaunchKernelGGL((linear_scan_kernel<PASS, LPC, CPL, false, true>), grid, block, smem, stream, a);     \
+  else if (PASS == 0 && bonus != nullptr)                                                                    \
+    hipLaunchKernelGGL((linear_scan_kernel<PASS, LPC, CPL, true, false>), grid, block, smem, stream, a);     \
   else                                                                                                       \
-    hipLaunchKernelGGL((linear_scan_kernel<PASS, LPC, CPL, false>), grid, block, smem, stream, a)
+    hipLaunchKernelGGL((linear_scan_kernel<PASS, LPC, CPL, false, false>), grid, block, smem, stream, a)
 #define ATOM_SCAN_BY_LPC(PASS, CPL)                       \
   switch (lpc) {                                          \
     case 1: ATOM_SCAN_LAUNCH(PASS, 1, CPL); break;        \

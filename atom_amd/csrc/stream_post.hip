@@ -192,6 +192,44 @@ ATOM_EXPORT int atom_rmsnorm_rows(const float* x, const float* weight, float eps
   return launch_status();
 }
 
+// stream[r] = (init ? 0 : stream[r]) + x[r] for float32 rows, and out[r] = norm(stream[r]) * weight in out's type: a
+// float32 summand (an embedding's output) starts the stream or joins it, and the stream is normed for the sublayer
+// that reads it next.  A block a row, the row's sum kept in LDS between the two walks.
+template <typename TO>
+__global__ void __launch_bounds__(256)
+stream_norm_kernel(float* __restrict__ stream, const float* __restrict__ x, const float* __restrict__ weight, float eps,
+                   TO* __restrict__ out, int width, int init) {
+  extern __shared__ float smem[];
+  float* vals = smem;
+  float* scratch = smem + width;
+  const size_t r = blockIdx.x;
+  float* sr = stream + r * width;
+  const float* xr = x + r * width;
+  float ss = 0.f;
+#pragma unroll 4
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float v = init ? xr[i] : sr[i] + xr[i];
+    sr[i] = v;
+    vals[i] = v;
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.f / sqrtf(ss / (float)width + eps);
+#pragma unroll 4
+  for (int i = threadIdx.x; i < width; i += blockDim.x) out[r * width + i] = from_f32<TO>(vals[i] * inv * weight[i]);
+}
+
+ATOM_EXPORT int atom_stream_norm(float* stream_rows, const float* x, const float* weight, float eps, void* out, int out_dtype,
+                                 int num_rows, int width, int init, hipStream_t stream) {
+  if (num_rows < 0 || width <= 0 || stream_rows == nullptr || x == nullptr || weight == nullptr || out == nullptr) return ATOM_BAD_SHAPE;
+  if (width > 32768) return ATOM_TOO_LARGE;
+  if (num_rows == 0) return ATOM_OK;
+  const size_t smem = (size_t)(width + 16) * sizeof(float);
+  ATOM_DISPATCH_DTYPE(out_dtype, hipLaunchKernelGGL((stream_norm_kernel<T>), dim3(num_rows), dim3(256), smem, stream,
+                                                     stream_rows, x, weight, eps, (T*)out, width, init));
+  return launch_status();
+}
+
 template <typename TO>
 __global__ void cast_rows_kernel(const float* __restrict__ x, TO* __restrict__ out, size_t n) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;

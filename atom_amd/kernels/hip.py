@@ -197,7 +197,8 @@ class HipKernels:
                    "atom_cast_rows", "atom_token_gate", "atom_embedding_bigram", "atom_rglru_scan",
                    "atom_keys_as_values_write", "atom_sigmoid_gate", "atom_bias_rows", "atom_linear_scan", "atom_token_shift",
                    "atom_step_decay", "atom_group_norm_gate", "atom_qkv_plain_write", "atom_narrow_heads",
-                   "atom_mean_of_norms", "atom_embedding_positions", "atom_unary_act", "atom_stream_add", "atom_scale_rows"):
+                   "atom_mean_of_norms", "atom_embedding_positions", "atom_unary_act", "atom_stream_add", "atom_scale_rows",
+                   "atom_stream_norm"):
             getattr(self.lib, fn).restype = ctypes.c_int
         self.allow_library_gemm = True
         # bfloat16 products of few rows run this library's own weight-streaming kernels: up to 64 rows, and
@@ -1183,14 +1184,16 @@ class HipKernels:
     def linear_scan(self, r, r_off: int, r_heads: int, k, k_off: int, k_heads: int, v, v_off: int, w, w_off: int,
                     state, state_off: int, cu_seqlens_q, slot_of_seq, out, heads: int, dim: int, vdim: int,
                     per_channel: bool = True, w_bias=None, v_scale=None, bonus=None, skip=None,
-                    max_q_len: int | None = None):
+                    max_q_len: int | None = None, step_bias=None, a_log=None):
         """A linear recurrence with a state of ``dim`` x ``vdim`` per head over each request's tokens:
         ``S <- diag(w) S + k v^T`` with the read-out ``o = (S_before + diag(bonus) k v^T)^T r`` where ``bonus``
         [heads, dim] is given, else ``o = S_after^T r``.  All inputs float32 [tokens, *], read from a column offset:
         ``r`` and ``k`` hold ``r_heads`` / ``k_heads`` heads of ``dim`` entries (head h reads head
         ``h // (heads / r_heads)``), ``v`` ``heads`` x ``vdim``, ``w`` the decays, ``heads`` x ``dim`` with
         ``per_channel`` and else one per head; with ``w_bias`` [heads, dim] the decay is ``exp(-exp(w + w_bias))``.
-        ``v_scale`` [tokens, heads] multiplies v on its way into the state; ``skip`` [heads] adds ``skip * v`` (v as
+        With ``a_log`` [heads] and ``step_bias`` [heads] (one decay per head) ``w`` holds raw step sizes:
+        ``step = softplus(w + step_bias)`` multiplies v on its way into the state and the decay is
+        ``exp(-exp(a_log) step)``.  ``v_scale`` [tokens, heads] multiplies v on its way into the state; ``skip`` [heads] adds ``skip * v`` (v as
         given) to the read-out.  The heads' matrices [heads, dim, vdim] start at ``state_off`` of a slot's row of
         ``state``; requests with slot -1 are padding.  ``out`` float32 [tokens, heads * vdim].  ``max_q_len``: the most tokens a
         request brings (an upper bound; default: all tokens); beyond ``SCAN_RUN`` tokens requests are cut into runs of
@@ -1212,6 +1215,13 @@ class HipKernels:
             self._check("decay bias", w_bias, torch.float32, (heads * dim,))
         if v_scale is not None:
             self._check("step sizes", v_scale, torch.float32, (tokens, heads))
+        mode, bias = (1, w_bias) if w_bias is not None else (0, None)
+        if a_log is not None:
+            if per_channel or w_bias is not None or v_scale is not None or bonus is not None or step_bias is None:
+                raise KernelError("linear_scan: raw step sizes go with one decay per head, a step bias and nothing else")
+            self._check("A_log", a_log, torch.float32, (heads,))
+            self._check("step bias", step_bias, torch.float32, (heads,))
+            mode, bias = 2, step_bias
         if bonus is not None:
             self._check("bonus", bonus, torch.float32, (heads, dim))
         if skip is not None:
@@ -1226,8 +1236,8 @@ class HipKernels:
             run_decay = torch.empty((places, heads, dim), dtype=torch.float32, device=out.device)
         self._done("linear_scan", self.lib.atom_linear_scan(
             self._at(r, r_off), L(r.shape[1]), heads // r_heads, self._at(k, k_off), L(k.shape[1]), heads // k_heads,
-            self._at(v, v_off), L(v.shape[1]), self._at(w, w_off), L(w.shape[1]), int(bool(per_channel)), _ptr(w_bias),
-            1 if w_bias is not None else 0, _ptr(v_scale), L(heads), _ptr(bonus), _ptr(skip), _ptr(out),
+            self._at(v, v_off), L(v.shape[1]), self._at(w, w_off), L(w.shape[1]), int(bool(per_channel)), _ptr(bias),
+            mode, _ptr(a_log), _ptr(v_scale), L(heads), _ptr(bonus), _ptr(skip), _ptr(out),
             L(heads * vdim), _ptr(state), L(state.shape[1]), L(state_off), _ptr(cu_seqlens_q), _ptr(slot_of_seq), seqs,
             heads, dim, vdim, tokens, run_len, _ptr(run_state), _ptr(run_decay), L(places), self._stream()))
         return out
@@ -1418,6 +1428,19 @@ class HipKernels:
         self._done("rmsnorm_rows", self.lib.atom_rmsnorm_rows(
             _ptr(x), _ptr(weight), ctypes.c_float(eps), _ptr(rows), n, _ptr(out), self._code(out), n_out, width,
             self._stream()))
+        return out
+
+    def stream_norm(self, stream, x, weight, eps: float, out, init: bool = False):
+        """``stream += x`` (``init``: ``stream = x``) for float32 rows, and ``out = norm(stream) * weight`` in
+        ``out``'s type, one kernel."""
+        n, width = stream.shape
+        self._check("stream", stream, torch.float32, (n, width))
+        self._check("summand", x, torch.float32, (n, width))
+        self._check("norm weight", weight, torch.float32, (width,))
+        self._check("norm out", out, (torch.float32, torch.bfloat16), (n, width))
+        self._done("stream_norm", self.lib.atom_stream_norm(
+            _ptr(stream), _ptr(x), _ptr(weight), ctypes.c_float(eps), _ptr(out), self._code(out), n, width,
+            int(bool(init)), self._stream()))
         return out
 
     def stream_add(self, stream, x, init: bool = False):

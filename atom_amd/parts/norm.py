@@ -39,13 +39,11 @@ class RMSNorm(Norm):
         if isinstance(x, torch.Tensor) and x.dtype == torch.float32 and ctx.dtype != torch.float32:
             # a float32 summand (an embedding's output that starts the stream or joins it again) in a step of
             # another type: the sum is formed in the stream, which is then normed into the step's type
-            if residual is None:
+            init = residual is None
+            if init:
                 residual = torch.empty(tuple(x.shape), dtype=torch.float32, device=x.device)
-                ctx.ops.stream_add(residual, x, init=True)
-            else:
-                ctx.ops.stream_add(residual, x)
             out = torch.empty(tuple(x.shape), dtype=ctx.dtype, device=x.device)
-            return ctx.ops.rmsnorm_rows(residual, self.params["weight"], self.eps, None, out), residual
+            return ctx.ops.stream_norm(residual, x, self.params["weight"], self.eps, out, init=init), residual
         pending = getattr(ctx.ops, "pending_norm", None)
         if pending is not None and residual is not None:
             # a product that has not been launched takes the residual sum as its epilogue and leaves the norm

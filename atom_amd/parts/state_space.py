@@ -76,13 +76,11 @@ class StateSpaceMixer(Mixer):
         xbc = torch.empty((T, C), dtype=torch.float32, device=x.device)
         ops.conv_silu_state(proj, C, self.params["conv.weight"], cache.state, ctx.cu_seqlens_q, ctx.slot_of_seq, xbc,
                             max_q_len=ctx.max_q_len, bias=self.params["conv.bias"], activation="silu", x_offset=inner)
-        dt = torch.empty((T, H), dtype=torch.float32, device=x.device)
-        decay = torch.empty((T, H), dtype=torch.float32, device=x.device)
-        ops.step_decay(proj, inner + C, self.params["dt_bias"], self.params["A_log"], dt, decay)
         y = torch.empty((T, inner), dtype=torch.float32, device=x.device)
-        ops.linear_scan(xbc, inner + G * N, G, xbc, inner, G, xbc, 0, decay, 0, cache.state, self.conv_floats,
-                        ctx.cu_seqlens_q, ctx.slot_of_seq, y, H, N, V, per_channel=False, v_scale=dt,
-                        skip=self.params["D"], max_q_len=ctx.max_q_len)
+        # the raw step sizes are the product's last columns: the scan forms softplus(dt + dt_bias) and the decays
+        ops.linear_scan(xbc, inner + G * N, G, xbc, inner, G, xbc, 0, proj, inner + C, cache.state, self.conv_floats,
+                        ctx.cu_seqlens_q, ctx.slot_of_seq, y, H, N, V, per_channel=False, skip=self.params["D"],
+                        max_q_len=ctx.max_q_len, step_bias=self.params["dt_bias"], a_log=self.params["A_log"])
         out = torch.empty((T, inner), dtype=x.dtype, device=x.device)
         ops.group_norm_gate(y, self.norm_groups, self.params["norm.weight"], self.norm_eps, out, gate=proj, gate_off=0,
                             gate_first=True)

@@ -342,11 +342,19 @@ class PlainKernels:
         out.copy_((pr.rms(src.to(WIDE), eps) * weight.to(WIDE)).to(out.dtype))
         return out
 
+    def stream_norm(self, stream, x, weight, eps, out, init=False):
+        stream.copy_(x.to(torch.float32) if init else (stream.to(WIDE) + x.to(WIDE)).to(torch.float32))
+        out.copy_((pr.rms(stream.to(WIDE), eps) * weight.to(WIDE)).to(out.dtype))
+        return out
+
     # ---- linear recurrences with a matrix state, attention without rotation, and what stands around them
 
     def linear_scan(self, r, r_off, r_heads, k, k_off, k_heads, v, v_off, w, w_off, state, state_off, cu_seqlens_q,
                     slot_of_seq, out, heads, dim, vdim, per_channel=True, w_bias=None, v_scale=None, bonus=None,
-                    skip=None, max_q_len=None):
+                    skip=None, max_q_len=None, step_bias=None, a_log=None):
+        if a_log is not None:      # raw step sizes in w's place: the steps multiply v, the decays follow from them
+            steps = pl.softplus(w[:, w_off:w_off + heads].to(WIDE) + step_bias.to(WIDE))
+            w, w_off, v_scale = torch.exp(-torch.exp(a_log.to(WIDE)) * steps), 0, steps
         for b in range(slot_of_seq.numel()):
             lo, hi, slot = int(cu_seqlens_q[b]), int(cu_seqlens_q[b + 1]), int(slot_of_seq[b])
             if slot < 0:

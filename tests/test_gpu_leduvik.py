@@ -80,6 +80,15 @@ def test_activations_sums_and_constants(dtype):
     close(s, x.double(), torch.float32, "stream = x")
     ops.scale_rows(s, 0.37)
     close(s, 0.37 * x.double(), torch.float32, "constant")
+    # a float32 summand starts the stream or joins it, and the stream is normed in the step's type
+    first, w = rnd((7, 53), 3), 1 + rnd((53,), 4, 0.2)
+    for init in (True, False):
+        s = f32(stream)
+        out = torch.empty((7, 53), dtype=dtype, device=DEV)
+        ops.stream_norm(s, f32(first), f32(w), 2e-5, out, init=init)
+        want = first.double() if init else stream.double() + first.double()
+        close(s, want, torch.float32, "stream and summand")
+        close(out, pl.rms_norm(want, w.double(), 2e-5), dtype, "its norm")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -222,13 +231,18 @@ def test_state_space_recurrence_carries_its_state(H, G, N, V):
     for step, lens in enumerate([[45, 2], [1, 19], [70, 1], [256, 131], [64, 65]]):
         T = sum(lens)
         xbc = rnd((T, inner + 2 * G * N), 10 + step, 0.8)
-        dt = pl.softplus(rnd((T, H), 20 + step).double())
+        raw, dt_bias = rnd((T, 3 + H + 2), 20 + step, 2.0), rnd((H,), 5)
+        dt = pl.softplus(raw[:, 3:3 + H].double() + dt_bias.double())
         decay = torch.exp(-A.double() * dt)
         cu, cu_d, slot_d, _ = _batch(lens, slots)
         out = torch.empty((T, inner), dtype=torch.float32, device=DEV)
         x_d = f32(xbc)
-        ops.linear_scan(x_d, inner + G * N, G, x_d, inner, G, x_d, 0, f32(decay), 0, state, 11, cu_d, slot_d, out, H, N, V,
-                        per_channel=False, v_scale=f32(dt), skip=f32(D))
+        if step % 2:     # steps and decays given
+            ops.linear_scan(x_d, inner + G * N, G, x_d, inner, G, x_d, 0, f32(decay), 0, state, 11, cu_d, slot_d, out, H, N, V,
+                            per_channel=False, v_scale=f32(dt), skip=f32(D))
+        else:            # raw step sizes: the kernel forms softplus(raw + bias) and the decays itself
+            ops.linear_scan(x_d, inner + G * N, G, x_d, inner, G, x_d, 0, f32(raw), 3, state, 11, cu_d, slot_d, out, H, N, V,
+                            per_channel=False, skip=f32(D), step_bias=f32(dt_bias), a_log=f32(torch.log(A)))
         for i in range(2):
             a, b = cu[i], cu[i + 1]
             x, B, C = torch.split(xbc[a:b].double(), [inner, G * N, G * N], dim=-1)
