@@ -45,6 +45,7 @@ struct RowsParams {
   const float* g_next;   // residual: [n], the weight of the norm that follows
   int m, n, k, inter, out_f32, mode, ss_parts, kslice, per_wave, tiles;   // kslice: k of a slice; per_wave: slices a wave
   int cols;              // output columns of a block: 16, 12 or 8 (gate: 8 gate and 8 up rows)
+  long batch_x, batch_w, batch_y;   // plain, several products side by side (blockIdx.y): elements between their x, w and y
   int act;               // plain: an activation on the product (0 none, 1 SiLU, 2 ReLU, 3 tanh-GELU, 4 ReLU squared, 5 tanh)
   float eps;
 };
@@ -61,6 +62,11 @@ template <int MR, int CG>
 // (up to 4 rows: 128 registers, so that a CU holds two blocks of 8 waves)
 __global__ void __launch_bounds__(512, (MR > 4 ? 3 : 4)) gemm_rows_kernel(RowsParams p) {
   constexpr int COLS = 4 * CG;
+  if (blockIdx.y > 0) {   // one of several products side by side: its own x, w and y
+    p.x += (size_t)blockIdx.y * p.batch_x;
+    p.w += (size_t)blockIdx.y * p.batch_w;
+    p.y = reinterpret_cast<char*>(p.y) + (size_t)blockIdx.y * p.batch_y * (p.out_f32 ? 4 : 2);
+  }
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int AREA = kRowsAWave + MR * kRowsA;
   constexpr int XJ = MR > 4 ? 2 : 1;     // 16-byte pieces of x a lane brings per quarter
@@ -272,7 +278,8 @@ ATOM_EXPORT int atom_gemm_rows_supports(int m, int n, int k) {
 }
 
 // mode 0 (plain): y [m, n], bfloat16 or float32 (out_f32), act(product + bias) with act 1 SiLU, 2 ReLU, 3 tanh-GELU,
-// 4 the square of ReLU, 5 tanh (0: none).   mode 1 (gate): w is [2 n, k], y [m, n] bfloat16.
+// 4 the square of ReLU, 5 tanh (0: none); `batch` > 1: that many products of the same sizes side by side, product b
+// reading x + b batch_x and w + b batch_w and writing y + b batch_y (elements; no bias, row choice or pending norm).   mode 1 (gate): w is [2 n, k], y [m, n] bfloat16.
 // mode 2 (residual): res [m, n] float32 += product, ss_out [m, atom_gemm_rows_parts(n, cols)], and, with g_next [n],
 // xg_out [m, n] = bf16(res * g_next).
 // cols: output columns a block owns in modes 0 and 2: 16, or 12 or 8 for widths whose 16-column tiles would leave
@@ -283,9 +290,12 @@ ATOM_EXPORT int atom_gemm_rows_supports(int m, int n, int k) {
 ATOM_EXPORT int atom_gemm_rows(const void* x, const int* rows, const float* ss, int ss_parts, float eps, const void* w,
                                const float* bias, void* y, float* res, float* ss_out, void* xg_out,
                                const float* g_next, int m, int n, int k, int mode, int out_f32, int cols,
-                               int waves_override, int act, hipStream_t stream) {
+                               int waves_override, int act, int batch, long batch_x, long batch_w, long batch_y,
+                               hipStream_t stream) {
   if (m < 0 || n <= 0 || k <= 0 || mode < 0 || mode > 2) return ATOM_BAD_SHAPE;
   if (act < 0 || act > 5 || (act != 0 && mode != ROWS_PLAIN)) return ATOM_UNSUPPORTED;
+  if (batch < 1 || batch > 65535 || batch_x < 0 || batch_w < 0 || batch_y < 0) return ATOM_BAD_SHAPE;
+  if (batch > 1 && (mode != ROWS_PLAIN || rows || ss || bias || (batch_x % 8) || (batch_w % 8))) return ATOM_UNSUPPORTED;
   if (!rows_cols_ok(cols) || (mode == ROWS_GATE && cols != 16)) return ATOM_UNSUPPORTED;
   if (!atom_gemm_rows_supports(max(m, 1), n, k)) return ATOM_UNSUPPORTED;
   if (m == 0) return ATOM_OK;
@@ -302,6 +312,7 @@ ATOM_EXPORT int atom_gemm_rows(const void* x, const int* rows, const float* ss, 
   p.tiles = rows_tiles(n, mode, cols);
   p.cols = cols;
   p.act = act;
+  p.batch_x = batch_x; p.batch_w = batch_w; p.batch_y = batch_y;
   int waves = rows_waves(m, p.tiles, k);
   if (waves_override == 4 || waves_override == 8) waves = waves_override;
   // 8 slices of K (4 where K is shorter than 8 quarters): the same for every number of rows and of waves
@@ -313,7 +324,7 @@ ATOM_EXPORT int atom_gemm_rows(const void* x, const int* rows, const float* ss, 
   const int mr = m <= 1 ? 1 : (m <= 2 ? 2 : (m <= 4 ? 4 : 8));
   const size_t lds = (size_t)waves * (kRowsAWave + mr * kRowsA) + 64 + (size_t)waves * 2 * 16 * 17 * 4;
 #define GO_ROWS(MRV, CGV) \
-  hipLaunchKernelGGL((gemm_rows_kernel<MRV, CGV>), dim3(p.tiles), dim3(64 * waves), lds, stream, p)
+  hipLaunchKernelGGL((gemm_rows_kernel<MRV, CGV>), dim3(p.tiles, batch), dim3(64 * waves), lds, stream, p)
 #define GO_ROWS_COLS(MRV)              \
   switch (cols) {                      \
     case 8: GO_ROWS(MRV, 2); break;    \

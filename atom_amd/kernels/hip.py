@@ -441,7 +441,8 @@ class HipKernels:
             head = (_ptr(x), None, None, 0, ctypes.c_float(0.0))
         self._done("gemm_rows", self.lib.atom_gemm_rows(
             *head, _ptr(weight), _ptr(bias), _ptr(y), _ptr(res), _ptr(ss_out), _ptr(xg_out), _ptr(g_next), m, n, k,
-            mode, int(out_f32), 16 if mode == 1 else self.rows_cols(n), int(self.rows_waves), act, self._stream()))
+            mode, int(out_f32), 16 if mode == 1 else self.rows_cols(n), int(self.rows_waves), act, 1, ctypes.c_long(0),
+            ctypes.c_long(0), ctypes.c_long(0), self._stream()))
 
     def _rows_product(self, x, weight, bias, out_dtype):
         y = torch.empty((x.shape[0], weight.shape[0]), dtype=out_dtype, device=weight.device)
@@ -843,6 +844,25 @@ class HipKernels:
         up = self.linear(x, weight, bias, out_dtype=out_dtype)
         out = torch.empty(tuple(up.shape), dtype=up.dtype, device=up.device)
         return self.unary_act(up, out, activation)
+
+    def linear_side_by_side(self, xs, weights, out_dtype=None):
+        """``ys[b] = xs[b] @ weights[b].T`` for ``xs`` [B, rows, k] and ``weights`` [B, n, k]: one launch where the
+        few-rows product takes the sizes, else a product each."""
+        B, m, k = xs.shape
+        n = weights.shape[1]
+        out_dtype = out_dtype or xs.dtype
+        if weights.shape[0] != B or weights.shape[2] != k:
+            raise KernelError("linear_side_by_side: as many weights as inputs, of the inputs' inner size")
+        if m and B > 1 and xs.is_contiguous() and weights.is_contiguous() and self._rows_takes(xs[0], weights[0]):
+            self._check("linear input", xs, torch.bfloat16)
+            self._check("linear weight", weights, torch.bfloat16)
+            ys = torch.empty((B, m, n), dtype=out_dtype, device=xs.device)
+            self._done("gemm_rows", self.lib.atom_gemm_rows(
+                _ptr(xs), None, None, 0, ctypes.c_float(0.0), _ptr(weights), None, _ptr(ys), None, None, None, None, m, n, k,
+                0, int(out_dtype == torch.float32), self.rows_cols(n), int(self.rows_waves), 0, B, ctypes.c_long(m * k),
+                ctypes.c_long(n * k), ctypes.c_long(m * n), self._stream()))
+            return [ys[b] for b in range(B)]
+        return [self.linear(xs[b], weights[b], None, out_dtype=out_dtype) for b in range(B)]
 
     def linear_silu(self, x, weight, bias=None):
         """``silu(x @ Wg.T + bg) * (x @ Wu.T + bu)`` for ``weight`` = gate rows then up rows: one kernel

@@ -53,10 +53,8 @@ class TimeMixRecurrence(Mixer):
             raise ValueError("decay_rank is not known: name it, or load the model from a checkpoint whose tensors say it")
         return {
             **{f"mu.{s}": ParamSpec.single(f"{n['mu']}.{s}", (h,), kind="vector") for s in self.MIXES},
-            "r.weight": ParamSpec.single(n["r"], (c, h)),
-            "k.weight": ParamSpec.single(n["k"], (c, h)),
-            "v.weight": ParamSpec.single(n["v"], (c, h)),
-            "gate.weight": ParamSpec.single(n["gate"], (c, h)),
+            # r, k, v and the gate as the four blocks of rows of one array: each multiplies a mix of its own, side by side
+            "rkvg.weight": ParamSpec.stacked([(n["r"], c), (n["k"], c), (n["v"], c), (n["gate"], c)], (h,)),
             "decay1.weight": ParamSpec.single(n["decay1"], (self.decay_rank, h)),
             "decay2.weight": ParamSpec.single(n["decay2"], (c, self.decay_rank)),
             "decay.bias": ParamSpec.single(n["decay_bias"], (c,), kind="vector"),
@@ -76,8 +74,7 @@ class TimeMixRecurrence(Mixer):
         mixes = torch.empty((5, T, W), dtype=x.dtype, device=x.device)
         ops.token_shift(x, self.mu, mixes, cache.state, 0, ctx.cu_seqlens_q, ctx.slot_of_seq, ctx.token_seq)
         # each of r, k, v and the gate reads a mix of its own
-        r, k, v, g = (ops.linear(mixes[i], self.params[f"{name}.weight"], None, out_dtype=torch.float32)
-                      for i, name in enumerate(("r", "k", "v", "gate")))
+        r, k, v, g = ops.linear_side_by_side(mixes[:4], self.params["rkvg.weight"].view(4, c, W), out_dtype=torch.float32)
         squashed = ops.linear_act(mixes[4], self.params["decay1.weight"], None, "tanh", out_dtype=torch.float32)
         raw = torch.empty((T, c), dtype=torch.float32, device=x.device)
         ops.heads_gemm(squashed, 0, rank, 0, self.params["decay2.weight"].view(1, c, rank), raw, 0, c, 0, 1, T, c, rank,

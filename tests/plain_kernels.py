@@ -114,6 +114,9 @@ class PlainKernels:
             y = y + bias.to(WIDE)
         return y.to(out_dtype or x.dtype)
 
+    def linear_side_by_side(self, xs, weights, out_dtype=None):
+        return [self.linear(xs[b], weights[b], None, out_dtype=out_dtype) for b in range(xs.shape[0])]
+
     def linear_act(self, x, weight, bias, activation, out_dtype=None):
         up = self.linear(x, weight, bias, out_dtype=WIDE)
         return self.unary_act(up, torch.empty(tuple(up.shape), dtype=out_dtype or x.dtype), activation)

@@ -108,6 +108,24 @@ def test_product_with_its_activation(dtype, rows):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows", [1, 5, 8, 70])
+def test_products_side_by_side(dtype, rows):
+    """Four products, each of an input of its own with a weight of its own: one launch for few rows, a product each
+    otherwise."""
+    ops = gpu_ops()
+    k, n = 192, 288
+    xs, ws = rnd((4, rows, k), 1).to(dtype), rnd((4, n, k), 2, k ** -0.5).to(dtype)
+    got = ops.linear_side_by_side(xs.to(DEV), ws.to(DEV), out_dtype=torch.float32)
+    assert len(got) == 4
+    for b in range(4):
+        assert got[b].dtype == torch.float32 and tuple(got[b].shape) == (rows, n)
+        close(got[b], xs[b].double() @ ws[b].double().T, torch.float32 if dtype == torch.float32 else dtype, f"product {b}")
+    same = ops.linear_side_by_side(xs.to(DEV), ws.to(DEV))
+    assert same[0].dtype == dtype
+    close(same[3], xs[3].double() @ ws[3].double().T, dtype, "in the inputs' type")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("width,n", [(40, 2), (192, 3), (1000, 1), (4096, 2)])
 def test_mean_of_normed_branches(dtype, width, n):
     ops = gpu_ops()
