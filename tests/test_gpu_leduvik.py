@@ -113,7 +113,7 @@ def test_products_side_by_side(dtype, rows):
     """Four products, each of an input of its own with a weight of its own: one launch for few rows, a product each
     otherwise."""
     ops = gpu_ops()
-    k, n = 192, 288
+    k, n = 160, 272
     xs, ws = rnd((4, rows, k), 1).to(dtype), rnd((4, n, k), 2, k ** -0.5).to(dtype)
     got = ops.linear_side_by_side(xs.to(DEV), ws.to(DEV), out_dtype=torch.float32)
     assert len(got) == 4
@@ -126,7 +126,7 @@ def test_products_side_by_side(dtype, rows):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("width,n", [(40, 2), (192, 3), (1000, 1), (4096, 2)])
+@pytest.mark.parametrize("width,n", [(40, 2), (176, 3), (1000, 1), (4096, 2)])
 def test_mean_of_normed_branches(dtype, width, n):
     ops = gpu_ops()
     eps = 2e-5
@@ -206,13 +206,13 @@ def test_step_sizes_and_decays():
     close(decay, torch.exp(-torch.exp(a_log.double()) * want), torch.float32, "decay")
 
 
-@pytest.mark.parametrize("H,K", [(5, 8), (2, 20), (6, 48), (2, 64), (1, 128), (3, 200)])
+@pytest.mark.parametrize("H,K", [(5, 8), (2, 20), (3, 48), (2, 64), (1, 128), (3, 200)])
 @pytest.mark.parametrize("lens", [[37, 1, 5], [3, 70, 1], [200, 64, 129], [128, 1, 65]])
 def test_time_mix_recurrence_carries_its_state(H, K, lens):
     """The bonus recurrence over three requests in two steps against the plain token-by-token form; the state of a
     request travels in its slot, a padding request between them touches nothing."""
     ops = gpu_ops()
-    T2 = [9, 4, 20] if lens[0] < 100 else [1, 192, 70]      # beyond 64 tokens a request is worked in runs side by side
+    T2 = [9, 4, 20] if lens[0] < 100 else [1, 193, 70]      # beyond 64 tokens a request is worked in runs side by side
     bonus, bias = rnd((H, K), 1, 0.5), rnd((H * K,), 2) - 1.0
     state = torch.zeros((5, 7 + H * K * K), dtype=torch.float32, device=DEV)
     slots = [3, 0, 4]
@@ -236,7 +236,7 @@ def test_time_mix_recurrence_carries_its_state(H, K, lens):
     assert float(state[:, :7].abs().max()) == 0 and float(state[1].abs().max()) == 0 and float(state[2].abs().max()) == 0
 
 
-@pytest.mark.parametrize("H,G,N,V", [(4, 2, 5, 6), (3, 1, 20, 12), (6, 1, 32, 48), (4, 4, 64, 32), (2, 1, 128, 64), (8, 2, 16, 100)])
+@pytest.mark.parametrize("H,G,N,V", [(4, 2, 5, 6), (3, 1, 20, 12), (6, 2, 32, 40), (4, 4, 64, 32), (2, 1, 128, 64), (8, 2, 16, 100)])
 def test_state_space_recurrence_carries_its_state(H, G, N, V):
     """Step sizes on the way into the state, one decay per head, groups of heads that share B and C, the skip
     weight on the read-out; x, B and C are columns of one array, as the convolution leaves them."""
@@ -303,7 +303,7 @@ def test_a_token_far_back_stays_in_the_states():
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("groups,gw", [(1, 40), (5, 8), (3, 100), (2, 256), (1, 288), (2, 1500), (1, 4096)])
+@pytest.mark.parametrize("groups,gw", [(1, 40), (5, 8), (3, 100), (2, 256), (1, 296), (2, 1500), (1, 4096)])
 @pytest.mark.parametrize("gate_first", [True, False])
 @pytest.mark.parametrize("off,pad", [(5, 3), (8, 4)])
 def test_norm_in_parts_with_a_gate(dtype, groups, gw, gate_first, off, pad):
@@ -321,7 +321,7 @@ def test_norm_in_parts_with_a_gate(dtype, groups, gw, gate_first, off, pad):
     close(out, want, dtype)
 
 
-@pytest.mark.parametrize("taps,channels,off", [(2, 24, 7), (3, 352, 288), (4, 300, 0), (5, 20, 3)])
+@pytest.mark.parametrize("taps,channels,off", [(2, 24, 7), (3, 344, 280), (4, 300, 0), (5, 20, 3)])
 def test_convolution_reads_its_columns_of_a_wider_product(taps, channels, off):
     """x | B | C are columns ``off .. off + channels`` of the packed product; the last ``taps - 1`` inputs travel in
     the slot and zeros stand before a request's start."""
@@ -388,7 +388,7 @@ def _write_and_attend(ops, proj, caches, order, page, a, b, H, G, D, V, DP, dtyp
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,G,D,V,DP,page,window,unit,temp", [
     (4, 2, 10, 6, 16, 4, 9, True, None), (6, 3, 6, 10, 16, 16, None, False, (0.25, 7)),
-    (4, 1, 64, 128, 128, 16, None, False, (0.3, 64)), (6, 2, 64, 64, 64, 16, 72, True, None),
+    (4, 2, 64, 128, 128, 16, None, False, (0.2, 48)), (6, 3, 64, 64, 64, 16, 80, True, None),
     (3, 3, 24, 40, 64, 8, 16, True, (0.5, 5)), (2, 1, 128, 32, 128, 16, 200, False, None)])
 def test_attention_with_unit_heads_temperature_and_window(dtype, H, G, D, V, DP, page, window, unit, temp):
     """A whole prompt, a portion behind cached keys and single tokens against the plain attention over the same
@@ -421,7 +421,7 @@ def test_attention_with_unit_heads_temperature_and_window(dtype, H, G, D, V, DP,
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("D,V,DP,page,window", [(64, 64, 64, 16, 72), (10, 6, 16, 4, 9), (32, 128, 128, 16, 16), (64, 32, 64, 16, 200)])
+@pytest.mark.parametrize("D,V,DP,page,window", [(64, 64, 64, 16, 80), (10, 6, 16, 4, 9), (32, 128, 128, 16, 16), (64, 32, 64, 16, 200)])
 def test_a_key_that_stands_out_is_seen_inside_the_window_only(dtype, D, V, DP, page, window):
     """One key among hundreds has a score far above the rest and a value like no other.  The query ``window - 1``
     places after it still returns its value, the next one does not; in prompts and for single tokens; the key right
@@ -452,16 +452,16 @@ def test_a_key_that_stands_out_is_seen_inside_the_window_only(dtype, D, V, DP, p
 def test_a_far_key_is_found_without_a_window(dtype):
     """Causal attention over everything: the key at position 2 of 900 is what the last query returns, decoded too."""
     ops = gpu_ops()
-    H, G, D, V, DP, page, n = 4, 1, 64, 128, 128, 16, 900
+    H, G, D, V, DP, page, n = 4, 2, 64, 128, 128, 16, 900
     proj = rnd((n, H * D + G * D + G * V), 4, 0.05)
     proj[:, 9:H * D:D] = 0.0                                   # no other query looks along entry 9
     proj[n - 1, :H * D] = 0.0
     proj[n - 1, 9:H * D:D] = 1.0
-    proj[2, H * D:H * D + D] = 0.0
-    proj[2, H * D + 9] = 60.0
-    proj[2, H * D + D:] = -5.0
+    proj[2, H * D:H * D + G * D] = 0.0
+    proj[2, H * D + 9:H * D + G * D:D] = 60.0
+    proj[2, H * D + G * D:] = -5.0
     k_cache, v_cache, order = _paged(torch.zeros(n, G, DP), None, page, dtype, order_seed=3)
-    args = (H, G, D, V, DP, dtype, False, 1e-6, (0.3, 64), 1.0, None)
+    args = (H, G, D, V, DP, dtype, False, 1e-6, (0.2, 50), 1.0, None)
     whole = _write_and_attend(ops, proj, (k_cache, v_cache), order, page, 0, n, *args)
     assert abs(float(whole[n - 1].float().mean()) + 5.0) < 0.1 and abs(float(whole[n - 2].float().mean())) < 1.0
     one = _write_and_attend(ops, proj, (k_cache, v_cache), order, page, n - 1, n, *args)
