@@ -435,10 +435,12 @@ class LeduvikConfig(ModelConfig):
 
     @classmethod
     def from_dict(cls, raw: dict) -> "LeduvikConfig":
-        layers = _need(raw, "layers", list, "the model")
+        layers = [cls._with_defaults(layer) for layer in _need(raw, "layers", list, "the model")]
         loop = raw.get("loop")
         if loop is not None:
             loop = tuple(_need(loop, k, int, "'loop'") for k in ("start", "stop", "times"))
+            if loop[0] == loop[1] or loop[2] == 1:
+                loop = None           # an empty run of layers, or a single pass: nothing is repeated
         cfg = cls(
             architecture=raw.get("architecture") or (raw.get("architectures") or ["Leduvik"])[0],
             vocab_size=_need(raw, "vocab", int, "the model"),
@@ -456,6 +458,32 @@ class LeduvikConfig(ModelConfig):
         )
         cfg.validate()
         return cfg
+
+    @staticmethod
+    def _with_defaults(layer):
+        """A layer's entry with the sizes that have an obvious value where the file leaves them out: as many
+        key/value heads as query heads, values of the keys' size, one group, one norm part."""
+        if not isinstance(layer, dict) or not isinstance(layer.get("mixer"), dict):
+            return layer
+
+        def attention(m):
+            m = dict(m)
+            if "heads" in m:
+                m.setdefault("kv_heads", m["heads"])
+            if "dim" in m:
+                m.setdefault("vdim", m["dim"])
+            return m
+
+        layer, m = dict(layer), dict(layer["mixer"])
+        if layer.get("type") == "mamba2":
+            m.setdefault("groups", 1)
+            m.setdefault("norm_groups", 1)
+        elif layer.get("type") == "attention":
+            m = attention(m)
+        elif layer.get("type") == "parallel" and isinstance(m.get("left"), dict):
+            m["left"] = attention(m["left"])
+        layer["mixer"] = m
+        return layer
 
     def validate(self) -> None:
         if self.vocab_size <= 0 or self.hidden_size <= 0 or not self.layers:

@@ -143,6 +143,21 @@ def test_names_and_shapes_are_the_designs(which):
                 assert branch.decay_rank == lt.RANKS[which]
 
 
+def test_sizes_left_out_take_their_obvious_values():
+    """No kv_heads: as many as heads; no vdim: the keys' size; no groups or norm_groups: one; a loop over no layers
+    or of one pass repeats nothing."""
+    raw = copy.deepcopy(lt.LEDU_B)
+    full = model_config_from_dict(raw)
+    del raw["layers"][0]["mixer"]["kv_heads"], raw["layers"][0]["mixer"]["vdim"], raw["layers"][1]["mixer"]["groups"]
+    assert model_config_from_dict(raw).layers == full.layers
+    raw["layers"][1]["mixer"].pop("norm_groups")
+    assert model_config_from_dict(raw).layers[1]["mixer"]["norm_groups"] == 1
+    for loop in ({"start": 2, "stop": 2, "times": 3}, {"start": 0, "stop": 3, "times": 1}):
+        raw["loop"] = loop
+        cfg = model_config_from_dict(raw)
+        assert cfg.loop is None and [r.layer for r in build_model(cfg).order] == [0, 1, 2, 3]
+
+
 def test_rank_without_a_checkpoint_must_be_named():
     with pytest.raises(ValueError, match="decay_rank"):
         expected_tensors(build_model(model_config_from_dict(lt.LEDU_A)))
