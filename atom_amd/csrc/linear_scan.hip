@@ -151,7 +151,13 @@ linear_scan_kernel(ScanArgs a) {
   const float skip = a.skip != nullptr ? a.skip[h] : 0.f;
   const int rh = h / a.r_div, kh = h / a.k_div;
 
-  for (int base = t0; base < t1; base += kStage) {
+  // One decay per head, first pass: B = sum_t (prod_{s > t} w_s) k_t (dt_t v_t)^T is formed from the run's last token
+  // to its first with the product of the decays behind a token as a factor on its v: one multiply-add a (row, column).
+  constexpr bool kBackward = PASS == 1 && PERHEAD;
+  float behind = 1.f;                        // kBackward: the product of the decays of the tokens already walked
+  const int stages = (t1 - t0 + kStage - 1) / kStage;
+  for (int st = 0; st < stages; ++st) {
+    const int base = t0 + (kBackward ? stages - 1 - st : st) * kStage;
     const int n = min(kStage, t1 - base);
     __syncthreads();
     // four entries a thread at a time, every load of the four asked for before the first is used
@@ -206,7 +212,8 @@ linear_scan_kernel(ScanArgs a) {
       staged[(size_t)j * per_token + NW * KP + c] = x;
     }
     __syncthreads();
-    for (int j = 0; j < n; ++j) {
+    for (int jj = 0; jj < n; ++jj) {
+      const int j = kBackward ? n - 1 - jj : jj;
       const float* src = staged + (size_t)j * per_token;
       const float4* r4 = reinterpret_cast<const float4*>(src + row0);
       const float4* k4 = reinterpret_cast<const float4*>(src + KP + row0);
@@ -219,6 +226,21 @@ linear_scan_kernel(ScanArgs a) {
         v_raw[c] = src[NW * KP + vcol + c];
         v[c] = v_raw[c] * step;
         acc[c] = 0.f;
+      }
+      if (kBackward) {
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) v[c] *= behind;
+        behind *= head_decay;
+#pragma unroll
+        for (int q = 0; q < kScanRows / 4; ++q) {
+          const float4 kq = k4[q];
+          const float kk[4] = {kq.x, kq.y, kq.z, kq.w};
+#pragma unroll
+          for (int x = 0; x < 4; ++x)
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) S[c][4 * q + x] = fmaf(kk[x], v[c], S[c][4 * q + x]);
+        }
+        continue;
       }
 #pragma unroll
       for (int q = 0; q < kScanRows / 4; ++q) {
@@ -268,6 +290,10 @@ linear_scan_kernel(ScanArgs a) {
     }
   }
   if (PASS == 1) {
+    if (kBackward) {
+#pragma unroll
+      for (int i = 0; i < kScanRows; ++i) u[i] = behind;   // every row of the head decays alike
+    }
 #pragma unroll
     for (int i = 0; i < kScanRows; ++i)
 #pragma unroll
