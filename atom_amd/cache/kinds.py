@@ -28,7 +28,7 @@ class KVBinding:
 
     group: int
     k_cache: torch.Tensor  # [num_pages, Hkv, page_size, D]
-    v_cache: torch.Tensor  # [num_pages, Hkv, D, page_size]
+    v_cache: torch.Tensor  # [num_pages, Hkv, D, page_size] (D: the value heads' size where it differs)
     writes: bool = True
 
 
@@ -111,11 +111,12 @@ class PagedKeysValues(CacheKind):
         return need.window is None and need.chunk is None
 
     def page_bytes(self, need, page_size, dtype):
-        return 2 * need.num_kv_heads * need.head_dim * page_size * _elem_size(dtype)
+        return need.num_kv_heads * (need.head_dim + (need.value_dim or need.head_dim)) * page_size * _elem_size(dtype)
 
     def allocate(self, need, *, group, num_pages, page_size, num_slots, device, dtype):
         k = torch.zeros((num_pages, need.num_kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
-        v = torch.zeros((num_pages, need.num_kv_heads, need.head_dim, page_size), dtype=dtype, device=device)
+        v = torch.zeros((num_pages, need.num_kv_heads, need.value_dim or need.head_dim, page_size), dtype=dtype,
+                        device=device)
         return KVBinding(group, k, v, writes=True)
 
     def share(self, binding):

@@ -1,9 +1,9 @@
 from .engine_config import Config
-from .model_config import (ConfigError, LotoraxConfig, ModelConfig, Qwen3Config, RalitarConfig,
+from .model_config import (ConfigError, LotoraxConfig, ModelConfig, Qwen3Config, RalitarConfig, SavidraConfig,
                            read_config_json)
 from .registry import (Architecture, build_model, get_architecture, known_architectures, model_config_from_dict,
                        register_architecture, unregister_architecture)
 
-__all__ = ["Config", "ConfigError", "ModelConfig", "Qwen3Config", "LotoraxConfig", "RalitarConfig", "read_config_json", "Architecture", "build_model",
+__all__ = ["Config", "ConfigError", "ModelConfig", "Qwen3Config", "LotoraxConfig", "RalitarConfig", "SavidraConfig", "read_config_json", "Architecture", "build_model",
            "get_architecture", "known_architectures", "model_config_from_dict", "register_architecture",
            "unregister_architecture"]

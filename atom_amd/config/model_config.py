@@ -555,6 +555,140 @@ class LeduvikConfig(ModelConfig):
         return out
 
 
+@dataclass(frozen=True)
+class SavidraConfig(ModelConfig):
+    """``Savidra``: token rows start a float32 stream that is normed after every sum, ``x <- norm(alpha x +
+    sublayer(x))``; the mixer reads a blend of a token's row and the previous token's; layers are listed one by
+    one, each softmax attention with a sink per head and values blended with an earlier layer's (``attention``)
+    or attention behind short convolutions, with a temperature per head and the heads' weights mixed, side by side
+    with a gated delta rule (``parallel``), and an optional ReLU-gated dense feed-forward.  config.json keys:
+    ``vocab``, ``width``, ``norm.eps``, ``postln_alpha``, ``layers`` (``type``, ``mixer``, ``mlp``)."""
+
+    layers: tuple = ()
+    norm_eps: float = 1e-6
+    postln_alpha: float = 1.0
+
+    model_type: ClassVar[str] = "savidra"
+    MIXER_TYPES: ClassVar[tuple] = ("attention", "parallel")
+    MLP_KINDS: ClassVar[tuple] = ("dense",)
+
+    @classmethod
+    def from_dict(cls, raw: dict) -> "SavidraConfig":
+        layers = [cls._with_defaults(layer) for layer in _need(raw, "layers", list, "the model")]
+        cfg = cls(
+            architecture=raw.get("architecture") or (raw.get("architectures") or ["Savidra"])[0],
+            vocab_size=_need(raw, "vocab", int, "the model"),
+            hidden_size=_need(raw, "width", int, "the model"),
+            num_hidden_layers=len(layers),
+            max_position_embeddings=_take(raw, "max_position_embeddings", int, 1 << 20),
+            tie_word_embeddings=False,
+            torch_dtype=str(raw.get("torch_dtype") or raw.get("dtype") or "bfloat16"),
+            bos_token_id=raw.get("bos_token_id"),
+            eos_token_id=raw.get("eos_token_id"),
+            layers=tuple(layers),
+            norm_eps=_need(raw.get("norm"), "eps", float, "'norm'"),
+            postln_alpha=_take(raw, "postln_alpha", float, 1.0),
+        )
+        cfg.validate()
+        return cfg
+
+    @staticmethod
+    def _with_defaults(layer):
+        """As many key/value heads as query heads and values of the keys' size where an entry leaves them out."""
+        if not isinstance(layer, dict) or not isinstance(layer.get("mixer"), dict):
+            return layer
+
+        def heads(m):
+            m = dict(m)
+            if "heads" in m:
+                m.setdefault("kv_heads", m["heads"])
+            if "dim" in m:
+                m.setdefault("vdim", m["dim"])
+            return m
+
+        layer, m = dict(layer), dict(layer["mixer"])
+        if layer.get("type") == "attention":
+            m = heads(m)
+        elif layer.get("type") == "parallel":
+            for side in ("left", "right"):
+                if isinstance(m.get(side), dict):
+                    m[side] = heads(m[side])
+        layer["mixer"] = m
+        return layer
+
+    def validate(self) -> None:
+        if self.vocab_size <= 0 or self.hidden_size <= 0 or not self.layers:
+            raise ConfigError("vocab, width and the number of layers must be positive")
+        if self.norm_eps <= 0:
+            raise ConfigError("norm.eps must be positive")
+
+        def positive(m, keys, where):
+            for key in keys:
+                if _need(m, key, int, where) <= 0:
+                    raise ConfigError(f"{where}: {key} must be positive")
+
+        def heads(m, where):
+            positive(m, ("heads", "kv_heads", "dim", "vdim"), where)
+            if m["heads"] % m["kv_heads"]:
+                raise ConfigError(f"{where}: heads must be a multiple of kv_heads")
+
+        def attention(m, where):
+            heads(m, where)
+            _need(m, "scale", float, where)
+            rot = m.get("rot")
+            if rot is not None:
+                dims = _need(rot, "dims", int, f"{where}'s rot")
+                _need(rot, "base", float, f"{where}'s rot")
+                if dims % 2 or dims < 0 or dims > m["dim"]:
+                    raise ConfigError(f"{where}: rot.dims must be even and at most dim")
+                if rot.get("scaling") is not None and _need(rot["scaling"], "factor", float, f"{where}'s rot.scaling") <= 0:
+                    raise ConfigError(f"{where}: rot.scaling.factor must be positive")
+            if m.get("conv") is not None and _need(m, "conv", int, where) <= 0:
+                raise ConfigError(f"{where}: conv must be positive")
+
+        mixed_values = None
+        for i, layer in enumerate(self.layers):
+            where = f"layer {i}"
+            kind = _need(layer, "type", str, where)
+            if kind not in self.MIXER_TYPES:
+                raise ConfigError(f"{where}: unknown type {kind!r}; known: {self.MIXER_TYPES}")
+            m = _need(layer, "mixer", dict, where)
+            mw = f"{where}'s mixer"
+            if kind == "attention":
+                attention(m, mw)
+                if m.get("v_mix"):
+                    size = m["kv_heads"] * m["vdim"]
+                    if mixed_values is not None and size != mixed_values:
+                        raise ConfigError(f"{where}: layers that blend their values need values of one size")
+                    mixed_values = size
+            else:
+                attention(_need(m, "left", dict, mw), f"{mw}'s left")
+                right = _need(m, "right", dict, mw)
+                heads(right, f"{mw}'s right")
+                positive(right, ("conv",), f"{mw}'s right")
+                for key in ("left_scale", "right_scale"):
+                    _need(m, key, float, mw)
+            mlp = layer.get("mlp")
+            if mlp is not None:
+                mk = _need(mlp, "kind", str, f"{where}'s mlp")
+                if mk not in self.MLP_KINDS:
+                    raise ConfigError(f"{where}: unknown mlp kind {mk!r}; known: {self.MLP_KINDS}")
+                positive(mlp, ("ff",), f"{where}'s mlp")
+
+    def to_dict(self) -> dict:
+        out: dict[str, Any] = {
+            "architecture": self.architecture, "model_type": self.model_type, "vocab": self.vocab_size,
+            "width": self.hidden_size, "norm": {"eps": self.norm_eps}, "postln_alpha": self.postln_alpha,
+            "layers": [dict(layer) for layer in self.layers],
+        }
+        if self.max_position_embeddings != 1 << 20:
+            out["max_position_embeddings"] = self.max_position_embeddings
+        for key in ("bos_token_id", "eos_token_id"):
+            if getattr(self, key) is not None:
+                out[key] = getattr(self, key)
+        return out
+
+
 def read_config_json(folder: str) -> dict:
     path = os.path.join(folder, "config.json")
     if not os.path.isfile(path):

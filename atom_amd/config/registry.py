@@ -7,7 +7,8 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Callable
 
-from .model_config import ConfigError, LeduvikConfig, LotoraxConfig, ModelConfig, Qwen3Config, RalitarConfig
+from .model_config import (ConfigError, LeduvikConfig, LotoraxConfig, ModelConfig, Qwen3Config, RalitarConfig,
+                           SavidraConfig)
 
 
 @dataclass(frozen=True)
@@ -83,3 +84,7 @@ def _ensure_builtin() -> None:
 
     if "Leduvik" not in _ARCHITECTURES:
         register_architecture("Leduvik", LeduvikConfig, leduvik_spec)
+    from ..models.savidra import savidra_spec
+
+    if "Savidra" not in _ARCHITECTURES:
+        register_architecture("Savidra", SavidraConfig, savidra_spec)

@@ -1,0 +1,193 @@
+// Paged softmax attention with the heads of a token worked through together: any head sizes (value heads may differ
+// from key heads), float32 or bfloat16, every query token of a mixed batch.
+//
+//   score_h(j) = (q_h . k_g(j)) * scale * head_scale[h]          (head_scale null: 1)
+//   w_h(j)     = exp(score_h(j) - m_h) / (sum_j' exp(score_h(j') - m_h) + exp(sink[h] - m_h))     (sink null: no such summand)
+//   w'_h(j)    = sum_g talk[h, g] w_g(j)                          (talk null: w' = w)
+//   out_h      = sum_j w'_h(j) v_{kv head of h}(j)
+//
+// A block owns one token and a set of heads: all of them when the heads' weights are mixed, else the query heads of
+// one key/value head.  Mixing needs the finished weights of all heads at a key, so the keys are walked twice: first
+// for every head's maximum and sum, then again for the weights themselves, their mixing and the weighted sum of the
+// values.  Keys are taken 64 at a time in chunks counted from position 0, so a token's result depends on its own
+// keys only: not on the batch, not on how a prompt was cut, not on which pages hold the keys.
+//
+// Pages: keys [pages, G, page, D]; values [pages, G, DV, page].
+#include "common.h"
+
+constexpr int kTogetherThreads = 256;
+constexpr int kTogetherChunk = 64;     // keys a pass; a wave's width, so a head's chunk is reduced by one wave
+constexpr int kTogetherAcc = 32;       // (head, value entry) pairs a thread may own
+
+struct TogetherArgs {
+  const int* token_seq; const int* positions; const int* block_tables; int max_blocks;
+  int H, G, D, DV, page_size, window;
+  float scale;
+  const float* head_scale; const float* sink; const float* talk;
+};
+
+// scores of the block's heads against the keys lo .. hi of a chunk that starts at base, into s[hb][kTogetherChunk]
+// (-inf outside lo .. hi)
+template <typename T>
+__device__ __forceinline__ void together_scores(const TogetherArgs& a, const T* __restrict__ k_cache, const int* table,
+                                                const float* qs, float* s, int h0, int HB, int base, int lo, int hi) {
+  const int group = a.H / a.G;
+  for (int item = threadIdx.x; item < HB * kTogetherChunk; item += kTogetherThreads) {
+    const int hh = item / kTogetherChunk, j = item - hh * kTogetherChunk;
+    const int key = base + j;
+    float v = -INFINITY;
+    if (key >= lo && key <= hi) {
+      const int h = h0 + hh;
+      const int page = table[key / a.page_size], off = key % a.page_size;
+      const T* kr = k_cache + (((size_t)page * a.G + h / group) * a.page_size + off) * (size_t)a.D;
+      const float* qr = qs + (size_t)hh * a.D;
+      float d = 0.f;
+      for (int i = 0; i < a.D; ++i) d += qr[i] * to_f32(kr[i]);
+      v = d * a.scale * (a.head_scale != nullptr ? a.head_scale[h] : 1.f);
+    }
+    s[item] = v;
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kTogetherThreads)
+attention_together_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                          T* __restrict__ out, TogetherArgs a) {
+  extern __shared__ float lds[];
+  const int t = blockIdx.x;
+  const int HB = a.talk != nullptr ? a.H : a.H / a.G;   // heads of this block
+  const int h0 = a.talk != nullptr ? 0 : blockIdx.y * HB;
+  float* qs = lds;                                  // HB * D
+  float* s = qs + (size_t)HB * a.D;                 // HB * chunk: scores, then weights
+  float* mixed = s + (size_t)HB * kTogetherChunk;   // HB * chunk: mixed weights (talk only)
+  float* top = mixed + (a.talk != nullptr ? (size_t)HB * kTogetherChunk : 0);   // HB: running maximum
+  float* den = top + HB;                            // HB: running sum, later its inverse
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1), wave = tid / kWave;
+  constexpr int waves = kTogetherThreads / kWave;
+  const int seq = a.token_seq[t];
+  const int items = HB * a.DV;
+  if (seq < 0) {   // padding row
+    for (int e = tid; e < items; e += kTogetherThreads) out[((size_t)t * a.H + h0) * a.DV + e] = from_f32<T>(0.f);
+    return;
+  }
+  const int pos = a.positions[t];
+  const int* table = a.block_tables + (size_t)seq * a.max_blocks;
+  for (int e = tid; e < HB * a.D; e += kTogetherThreads) qs[e] = to_f32(q[((size_t)t * a.H + h0) * a.D + e]);
+  for (int e = tid; e < HB; e += kTogetherThreads) top[e] = -INFINITY, den[e] = 0.f;
+  __syncthreads();
+  const int first = (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
+  const int start = first / kTogetherChunk * kTogetherChunk;
+
+  // every head's maximum and sum
+  for (int base = start; base <= pos; base += kTogetherChunk) {
+    const int lo = base > first ? base : first;
+    const int hi = base + kTogetherChunk - 1 < pos ? base + kTogetherChunk - 1 : pos;
+    together_scores(a, k_cache, table, qs, s, h0, HB, base, lo, hi);
+    __syncthreads();
+    for (int hh = wave; hh < HB; hh += waves) {     // a head is always the same wave's
+      const float v = s[hh * kTogetherChunk + lane];
+      const float m_old = top[hh];
+      const float m_new = fmaxf(m_old, wave_max(v));   // finite: a chunk holds at least one visible key
+      const float sum = wave_sum(expf(v - m_new));
+      if (lane == 0) {
+        den[hh] = den[hh] * (m_old == -INFINITY ? 0.f : expf(m_old - m_new)) + sum;
+        top[hh] = m_new;
+      }
+    }
+    __syncthreads();
+  }
+  for (int hh = tid; hh < HB; hh += kTogetherThreads) {
+    float m = top[hh], l = den[hh];
+    if (a.sink != nullptr) {
+      const float sk = a.sink[h0 + hh];
+      const float m_new = fmaxf(m, sk);
+      l = l * expf(m - m_new) + expf(sk - m_new);
+      m = m_new;
+    }
+    top[hh] = m;
+    den[hh] = 1.f / l;
+  }
+  __syncthreads();
+
+  // the weights, their mixing, the weighted sum of the values
+  float acc[kTogetherAcc];
+#pragma unroll
+  for (int r = 0; r < kTogetherAcc; ++r) acc[r] = 0.f;
+  const int group = a.H / a.G;
+  for (int base = start; base <= pos; base += kTogetherChunk) {
+    const int lo = base > first ? base : first;
+    const int hi = base + kTogetherChunk - 1 < pos ? base + kTogetherChunk - 1 : pos;
+    together_scores(a, k_cache, table, qs, s, h0, HB, base, lo, hi);
+    // a thread turns the scores it wrote itself into weights
+    for (int item = tid; item < HB * kTogetherChunk; item += kTogetherThreads) {
+      const int hh = item / kTogetherChunk;
+      s[item] = expf(s[item] - top[hh]) * den[hh];    // exp(-inf) = 0 outside lo .. hi
+    }
+    __syncthreads();
+    const float* w = s;
+    if (a.talk != nullptr) {
+      for (int item = tid; item < HB * kTogetherChunk; item += kTogetherThreads) {
+        const int hh = item / kTogetherChunk, j = item - hh * kTogetherChunk;
+        const float* row = a.talk + (size_t)hh * a.H;
+        float m = 0.f;
+        for (int g = 0; g < a.H; ++g) m += row[g] * s[g * kTogetherChunk + j];
+        mixed[item] = m;
+      }
+      __syncthreads();
+      w = mixed;
+    }
+#pragma unroll
+    for (int r = 0; r < kTogetherAcc; ++r) {
+      const int e = tid + r * kTogetherThreads;
+      if (e < items) {
+        const int hh = e / a.DV, i = e - hh * a.DV;
+        const int kvh = (h0 + hh) / group;
+        const float* wr = w + hh * kTogetherChunk - base;   // wr[key]
+        float sum = acc[r];
+        for (int key = lo; key <= hi;) {
+          const int page = table[key / a.page_size], off = key % a.page_size;
+          int run = a.page_size - off;
+          if (run > hi - key + 1) run = hi - key + 1;
+          const T* vr = v_cache + (((size_t)page * a.G + kvh) * a.DV + i) * (size_t)a.page_size + off;
+          for (int u = 0; u < run; ++u) sum += wr[key + u] * to_f32(vr[u]);
+          key += run;
+        }
+        acc[r] = sum;
+      }
+    }
+    __syncthreads();   // s and mixed are rewritten by the next chunk
+  }
+#pragma unroll
+  for (int r = 0; r < kTogetherAcc; ++r) {
+    const int e = tid + r * kTogetherThreads;
+    if (e < items) out[((size_t)t * a.H + h0) * a.DV + e] = from_f32<T>(acc[r]);
+  }
+}
+
+static size_t together_lds(int H, int G, int D, bool talk) {
+  const int HB = talk ? H : H / G;
+  return ((size_t)HB * D + (size_t)HB * kTogetherChunk * (talk ? 2 : 1) + 2 * (size_t)HB) * sizeof(float);
+}
+
+ATOM_EXPORT int atom_attention_together(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
+                                        const int* token_seq, const int* positions, const int* block_tables,
+                                        int max_blocks, int tokens, int H, int G, int D, int DV, int page_size,
+                                        float scale, const float* head_scale, const float* sink, const float* talk,
+                                        int window, hipStream_t stream) {
+  if (tokens < 0 || H <= 0 || G <= 0 || D <= 0 || DV <= 0 || page_size <= 0 || max_blocks <= 0) return ATOM_BAD_SHAPE;
+  if (H % G || window < 0) return ATOM_BAD_SHAPE;
+  if (q == nullptr || k_cache == nullptr || v_cache == nullptr || out == nullptr) return ATOM_BAD_SHAPE;
+  if (token_seq == nullptr || positions == nullptr || block_tables == nullptr) return ATOM_BAD_SHAPE;
+  const bool mixes = talk != nullptr;
+  const int HB = mixes ? H : H / G;
+  if ((size_t)HB * DV > (size_t)kTogetherAcc * kTogetherThreads) return ATOM_TOO_LARGE;
+  const size_t smem = together_lds(H, G, D, mixes);
+  if (smem > 64 * 1024) return ATOM_TOO_LARGE;
+  if (tokens == 0) return ATOM_OK;
+  TogetherArgs a{token_seq, positions, block_tables, max_blocks, H, G, D, DV, page_size, window, scale, head_scale, sink, talk};
+  dim3 grid(tokens, mixes ? 1 : G), block(kTogetherThreads);
+  ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((attention_together_kernel<T>), grid, block, smem, stream, (const T*)q,
+                                                 (const T*)k_cache, (const T*)v_cache, (T*)out, a));
+  return launch_status();
+}

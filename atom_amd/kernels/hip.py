@@ -198,7 +198,8 @@ class HipKernels:
                    "atom_keys_as_values_write", "atom_sigmoid_gate", "atom_bias_rows", "atom_linear_scan", "atom_token_shift",
                    "atom_step_decay", "atom_group_norm_gate", "atom_qkv_plain_write", "atom_narrow_heads",
                    "atom_mean_of_norms", "atom_embedding_positions", "atom_unary_act", "atom_stream_add", "atom_scale_rows",
-                   "atom_stream_norm"):
+                   "atom_stream_norm", "atom_sum_norm", "atom_shift_rows", "atom_qkv_rot_write",
+                   "atom_attention_together"):
             getattr(self.lib, fn).restype = ctypes.c_int
         self.allow_library_gemm = True
         # bfloat16 products of few rows run this library's own weight-streaming kernels: up to 64 rows, and
@@ -375,6 +376,10 @@ class HipKernels:
             out = torch.empty(tuple(x.shape), dtype=x.dtype, device=x.device)
             # the float32 rows as a sum of one slice: the norm kernel reads float32 and writes the step's type
             return self.rmsnorm(DeferredSum(x.r.unsqueeze(0), None, x.dtype), x.weight, x.eps, out, rows=x.rows)
+        if hasattr(x, "terms"):
+            # a sum of scaled terms that a mixer handed on, added up in float32
+            out = torch.empty(tuple(x.shape), dtype=torch.float32, device=x.device)
+            return self.sum_norm(out, 0.0, x.terms, x.scales, None, 0.0)
         if not isinstance(x, DeferredSum):
             return x
         rows, width = x.shape
@@ -1601,6 +1606,120 @@ class HipKernels:
         return out
 
     # ------------------------------------------------------------------ routed experts
+
+    # ------------------------------------------------------------------ a stream normed after every sum; heads together
+
+    def sum_norm(self, stream, alpha: float, summands, scales, weight, eps: float, out=None):
+        """``stream <- rms_norm(alpha * stream + sum_i scales[i] * summands[i]) * weight`` in float32, in place
+        (``weight`` None: the sum alone; ``alpha`` 0: the stream's old rows are not read); up to four summands of
+        float32 or bfloat16.  ``out``, when given, receives the new rows in its own type.  Returns ``stream``."""
+        rows, width = stream.shape
+        self._check("stream", stream, torch.float32, (rows, width))
+        summands = [self.materialize(y) for y in summands]
+        if len(summands) > 4 or len(summands) != len(scales):
+            raise KernelError("sum_norm: up to four summands, a scale each")
+        for y in summands:
+            self._check("summand", y, (torch.float32, torch.bfloat16), (rows, width))
+        if weight is not None:
+            self._check("norm weight", weight, torch.float32, (width,))
+        if out is not None:
+            self._check("stream copy", out, (torch.float32, torch.bfloat16), (rows, width))
+        terms = []
+        for i in range(4):
+            if i < len(summands):
+                terms += [_ptr(summands[i]), self._code(summands[i]), ctypes.c_float(scales[i])]
+            else:
+                terms += [None, 0, ctypes.c_float(0.0)]
+        self._done("sum_norm", self.lib.atom_sum_norm(
+            _ptr(stream), ctypes.c_float(alpha), *terms, len(summands), _ptr(weight), ctypes.c_float(eps), _ptr(out),
+            self._code(out) if out is not None else 0, rows, width, self._stream()))
+        return stream
+
+    def shift_rows(self, x, mu, out, state, state_off: int, cu_seqlens_q, slot_of_seq, token_seq):
+        """``out[t] = x[t] + (x[t - 1] - x[t]) * mu``; the row before a request's first token of the step is what its
+        state slot holds at ``state_off`` (float32, zeros for a fresh request), and the request's last row of the
+        step is left there.  ``x`` and ``out`` float32 or bfloat16, independently."""
+        tokens, width = x.shape
+        seqs = slot_of_seq.numel()
+        self._check("shift input", x, (torch.float32, torch.bfloat16))
+        self._check("shift weight", mu, torch.float32, (width,))
+        self._check("shifted rows", out, (torch.float32, torch.bfloat16), (tokens, width))
+        self._check("state", state, torch.float32, (None, None))
+        self._check("cu_seqlens_q", cu_seqlens_q, torch.int32, (seqs + 1,))
+        self._check("slot_of_seq", slot_of_seq, torch.int32, (seqs,))
+        self._check("token_seq", token_seq, torch.int32, (tokens,))
+        self._done("shift_rows", self.lib.atom_shift_rows(
+            _ptr(x), self._code(x), _ptr(mu), _ptr(out), self._code(out), _ptr(state), ctypes.c_long(state.shape[1]),
+            ctypes.c_long(state_off), _ptr(cu_seqlens_q), _ptr(slot_of_seq), _ptr(token_seq), tokens, width,
+            self._stream()))
+        return out
+
+    def qkv_rot_write(self, qkv, q_out, k_cache, v_cache, q_weight, k_weight, freq, rot_dims: int, positions, slots,
+                      num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, page_size: int, eps: float,
+                      v_source=None, v_blend=None, v_keep=None):
+        """From the float32 rows ``q | k | v`` of every token: RMS norm of every q and k head with a weight per
+        entry (None: no norm), rotation of the pairs (i, i + rot_dims / 2) of every head by ``position * freq[i]``
+        (``freq`` float64), ``v_keep`` (float32 [tokens, G * DV]) receives the values as they are, and with
+        ``v_source`` (float32, the same shape) the values become ``(1 - l) v + l v_source``, ``l = v_blend`` (one
+        float32 number on the device).  q goes to ``q_out`` [tokens, H, D], k to the key pages [pages, G, page, D],
+        v to the value pages [pages, G, DV, page] at ``slots`` (-1: no write)."""
+        tokens, ld = qkv.shape
+        H, G, D, DV = num_heads, num_kv_heads, head_dim, value_dim
+        self._check("q | k | v", qkv, torch.float32)
+        dt = q_out.dtype
+        self._check("q", q_out, (torch.float32, torch.bfloat16), (tokens, H, D))
+        self._check("key pages", k_cache, dt, (None, G, page_size, D))
+        self._check("value pages", v_cache, dt, (k_cache.shape[0], G, DV, page_size))
+        self._check("slot mapping", slots, torch.int32, (tokens,))
+        for name, w in (("q norm weight", q_weight), ("k norm weight", k_weight)):
+            if w is not None:
+                self._check(name, w, torch.float32, (D,))
+        if rot_dims:
+            self._check("rotation frequencies", freq, torch.float64, (rot_dims // 2,))
+            self._check("positions", positions, torch.int32, (tokens,))
+        for name, t in (("source values", v_source), ("kept values", v_keep)):
+            if t is not None:
+                self._check(name, t, torch.float32, (tokens, G * DV))
+        if v_source is not None:
+            self._check("blend", v_blend, torch.float32, ())
+        self._done("qkv_rot_write", self.lib.atom_qkv_rot_write(
+            _ptr(qkv), ld, _ptr(q_out), _ptr(k_cache), _ptr(v_cache), self._code(q_out), _ptr(q_weight), _ptr(k_weight),
+            _ptr(freq) if rot_dims else None, int(rot_dims), _ptr(positions) if rot_dims else None, _ptr(slots), tokens,
+            H, G, D, DV, page_size, ctypes.c_float(eps), _ptr(v_source), _ptr(v_blend) if v_source is not None else None,
+            _ptr(v_keep), self._stream()))
+        return q_out
+
+    def attention_together(self, q, k_cache, v_cache, out, token_seq, positions, block_tables, scale: float,
+                           head_scale=None, sink=None, talk=None, window: int | None = None,
+                           max_context_len: int | None = None):
+        """Softmax attention of the step's queries over the pages with a token's heads worked through together:
+        ``head_scale`` (float32 [H]) multiplies the scaled scores of a head, ``sink`` (float32 [H]) joins the
+        softmax's denominator as ``exp(sink[h])`` without a value, ``talk`` (float32 [H, H]) mixes the heads'
+        finished weights, ``w_h <- sum_g talk[h, g] w_g``, before head h applies them to the values of its own
+        key/value head.  Value heads [pages, G, DV, page] may differ in size from key heads [pages, G, page, D]."""
+        tokens, H, D = q.shape
+        _, G, page_size, _ = k_cache.shape
+        DV = v_cache.shape[2]
+        dt = q.dtype
+        self._check("q", q, (torch.float32, torch.bfloat16))
+        self._check("key pages", k_cache, dt, (None, G, page_size, D))
+        self._check("value pages", v_cache, dt, (k_cache.shape[0], G, DV, page_size))
+        self._check("attention out", out, dt, (tokens, H, DV))
+        self._check("token_seq", token_seq, torch.int32, (tokens,))
+        self._check("positions", positions, torch.int32, (tokens,))
+        self._check("block tables", block_tables, torch.int32, (None, None))
+        if max_context_len is not None and max_context_len > block_tables.shape[1] * page_size:
+            raise KernelError("attention: a context is longer than its block table can name")
+        for name, w in (("head scale", head_scale), ("sink", sink)):
+            if w is not None:
+                self._check(name, w, torch.float32, (H,))
+        if talk is not None:
+            self._check("head mixing", talk, torch.float32, (H, H))
+        self._done("attention_together", self.lib.atom_attention_together(
+            _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), self._code(q), _ptr(token_seq), _ptr(positions),
+            _ptr(block_tables), block_tables.shape[1], tokens, H, G, D, DV, page_size, ctypes.c_float(scale),
+            _ptr(head_scale), _ptr(sink), _ptr(talk), int(window or 0), self._stream()))
+        return out
 
     def router_choose(self, logits, correction, top: int, renormalize: bool = False):
         """(ids int32 [tokens, top], weights float32 [tokens, top]) from float32 router logits: scores are

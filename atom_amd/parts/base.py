@@ -58,6 +58,11 @@ class ParamSpec:
         return ParamSpec(tuple(shape), kind, (Source(name, 0, shape[0]),), init)
 
     @staticmethod
+    def scalar(name: str, kind: str = "vector", init: str = "normal") -> "ParamSpec":
+        """One number, stored as a tensor without dimensions."""
+        return ParamSpec((), kind, (Source(name, 0, 0),), init)
+
+    @staticmethod
     def stacked(names_rows: list[tuple[str, int]], trailing: tuple[int, ...], kind: str = "matrix",
                 init: str = "normal") -> "ParamSpec":
         sources, offset = [], 0
@@ -116,6 +121,7 @@ class KVCacheNeed:
     head_dim: int
     window: int | None = None
     chunk: int | None = None
+    value_dim: int | None = None    # entries of a value head where they differ from a key head's (None: head_dim)
 
 
 @dataclass(frozen=True)
@@ -136,6 +142,25 @@ class StateNeed:
 
 
 # ----------------------------------------------------------------------------- the four computing kinds
+
+
+class ScaledSum:
+    """What a mixer may return instead of a tensor: ``sum_i scales[i] * terms[i]`` (tensors of one shape, any types),
+    not yet added up.  A block whose norm takes several summands hands the terms on as they are; anything else calls
+    ``ops.materialize``, which adds them in float32."""
+
+    def __init__(self, terms: list, scales: list):
+        self.terms, self.scales = list(terms), [float(s) for s in scales]
+
+    @property
+    def shape(self):
+        return self.terms[0].shape
+
+    @property
+    def device(self):
+        return self.terms[0].device
+
+    dtype = torch.float32
 
 
 class Norm(Part):
@@ -191,6 +216,9 @@ class Mixer(Part):
     #: True when ``forward`` launches the same kernels whatever the batch holds and reads the batch
     #: only through device arrays of ``ctx``: a decode step of such mixers may be replayed as a HIP graph
     graph_safe = False
+    #: True when ``forward`` wants the float32 residual stream's rows themselves where a block keeps one, not
+    #: their copy in the step's type
+    reads_stream = False
 
     def cache_need(self):
         """What this mixer keeps between steps: a ``KVCacheNeed``, a ``StateNeed``, an object of any other

@@ -6,7 +6,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block, PartChoice
+from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block, PartChoice, ScaledSum
 
 
 class PreNormBlock(Block):
@@ -153,6 +153,65 @@ class PostNormBlock(Block):
         return stream, None
 
 
+class NormedSumBlock(Block):
+    """The norm comes after the sum and its result is the stream: ``x <- norm1(alpha x + mixer(x))``, then
+    ``x <- norm2(alpha x + ffn(x))`` (``feed_forward`` None leaves the second step out).  The sublayers read the
+    stream, which is float32 and kept whole (nothing pending); its rows in the step's type, for the products that
+    read them, come out of the kernel that norms it.  A mixer with ``reads_stream`` is handed the float32 rows.
+    ``names["mixer"]`` may be empty: the mixer then takes the layer's own prefix."""
+
+    def __init__(self, mixer: PartChoice, feed_forward: PartChoice | None, norm: PartChoice, alpha: float = 1.0,
+                 prefix: str = "", names: dict[str, str] | None = None):
+        super().__init__(prefix)
+        n = {"mixer": "mix", "mixer_norm": "norm1", "ffn": "mlp", "ffn_norm": "norm2", **(names or {})}
+        sub = lambda name: (f"{prefix}.{n[name]}" if prefix else n[name]) if n[name] else prefix  # noqa: E731
+        self.alpha = float(alpha)
+        self._mixer = mixer.build(MIXERS, prefix=sub("mixer"))
+        self.mixer_norm = norm.build(NORMS, prefix=sub("mixer_norm"))
+        self.ffn = feed_forward.build(FEED_FORWARDS, prefix=sub("ffn")) if feed_forward is not None else None
+        self.ffn_norm = norm.build(NORMS, prefix=sub("ffn_norm")) if self.ffn is not None else None
+        for post in (self.mixer_norm, self.ffn_norm):
+            if post is not None and not hasattr(post, "forward_sum"):
+                raise ValueError(f"{type(post).__name__} cannot norm a sum into the stream (no forward_sum)")
+
+    @property
+    def mixer(self):
+        return self._mixer
+
+    def children(self):
+        return [self._mixer, self.mixer_norm] + ([self.ffn, self.ffn_norm] if self.ffn is not None else [])
+
+    @staticmethod
+    def _summands(ops, y):
+        if isinstance(y, ScaledSum):
+            return [ops.materialize(t) for t in y.terms], y.scales
+        return [ops.materialize(y)], [1.0]
+
+    def forward(self, ctx, hidden, residual, cache):
+        ops = ctx.ops
+        if residual is not None:
+            raise ValueError("this block takes the whole stream, with nothing pending beside it")
+        stream = ops.materialize(hidden)
+        if stream.dtype != torch.float32:
+            raise ValueError("this block keeps a float32 stream: the embedding before it must write float32")
+        reads = ctx.memo.pop(("stream copy", stream.data_ptr()), None)
+        if self._mixer.reads_stream:
+            reads = stream
+        elif reads is None:
+            reads = stream if ctx.dtype == torch.float32 else ops.cast_rows(stream, ctx.dtype)
+        terms, scales = self._summands(ops, self._mixer.forward(ctx, reads, cache))
+        # the copy is for the feed-forward, or for the next block's mixer where that reads one
+        reads = self.mixer_norm.forward_sum(ctx, terms, scales, stream, self.alpha,
+                                            copy=self.ffn is not None or not self._mixer.reads_stream)
+        if self.ffn is not None:
+            terms, scales = self._summands(ops, self.ffn.forward(ctx, reads))
+            reads = self.ffn_norm.forward_sum(ctx, terms, scales, stream, self.alpha, copy=not self._mixer.reads_stream)
+        if reads is not stream:
+            ctx.memo[("stream copy", stream.data_ptr())] = reads
+        return stream, None
+
+
 BLOCKS.register("prenorm", PreNormBlock)
+BLOCKS.register("normed_sum", NormedSumBlock)
 BLOCKS.register("sandwich", SandwichBlock)
 BLOCKS.register("postnorm", PostNormBlock)

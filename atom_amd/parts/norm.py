@@ -13,14 +13,32 @@ from .base import NORMS, Norm, ParamSpec
 class RMSNorm(Norm):
     accepts_deferred = True   # the kernel adds the slices of a product that is still a sum
 
-    def __init__(self, size: int, eps: float, prefix: str = "", weight_name: str = "weight"):
+    def __init__(self, size: int, eps: float, prefix: str = "", weight_name: str = "weight", one_plus: bool = False):
         super().__init__(prefix)
         self.size = size
         self.eps = float(eps)
         self.weight_name = weight_name   # the checkpoint's name under the prefix (empty: the prefix itself)
+        self.one_plus = bool(one_plus)   # the checkpoint stores the weight's distance from one
+        self._folded = False
 
     def param_specs(self):
-        return {"weight": ParamSpec.single(self.weight_name, (self.size,), kind="vector", init="one_plus_normal")}
+        return {"weight": ParamSpec.single(self.weight_name, (self.size,), kind="vector",
+                                           init="normal" if self.one_plus else "one_plus_normal")}
+
+    def finalize(self, device, dtype):
+        if self.one_plus and not self._folded:
+            self.params["weight"] = 1.0 + self.params["weight"]    # float32
+            self._folded = True
+
+    def forward_sum(self, ctx, summands, scales, stream, alpha: float, copy: bool = True):
+        """``stream <- norm(alpha * stream + sum_i scales[i] * summands[i])`` in float32 (one or two summands of any
+        type, nothing rounded on the way); returns the stream's new rows in the step's type for the sublayer that
+        reads them next (``copy`` False, or a float32 step: the stream itself)."""
+        out = None
+        if copy and ctx.dtype != torch.float32:
+            out = torch.empty(tuple(stream.shape), dtype=ctx.dtype, device=stream.device)
+        ctx.ops.sum_norm(stream, float(alpha), summands, scales, self.params["weight"], self.eps, out)
+        return stream if out is None else out
 
     def forward_post(self, ctx, x, stream, copy: bool = True):
         """``stream += norm(x)`` in float32, nothing rounded on the way; returns the stream's rows in the step's

@@ -131,6 +131,33 @@ class BandedRotary(PositionEncoding):
         self.freq = self.frequencies().to(device)
 
 
+class HalfRotary(PositionEncoding):
+    """Rotation of the pairs (i, i + dims / 2) of the first ``dims`` entries of a head by ``position * f_i``,
+    ``f_i = base^(-2i / dims) / factor`` (``factor``: positions stretched linearly; None: 1).  Offers what
+    ``ScaledRotary`` offers (``freq`` float64 [dims / 2] on the device, ``mult``, ``dims``): kernels form the angle
+    in float64 from the position, so there is no table and no position limit."""
+
+    def __init__(self, dims: int, base: float, factor: float | None = None, head_dim: int | None = None,
+                 prefix: str = ""):
+        super().__init__(prefix)
+        if dims % 2 or dims < 0 or (head_dim is not None and dims > head_dim):
+            raise ValueError(f"rotated dimensions come in pairs within a head, got {dims}")
+        if factor is not None and not float(factor) > 0:
+            raise ValueError("the stretch of positions must be positive")
+        self.dims, self.base = int(dims), float(base)
+        self.factor = float(factor) if factor is not None else 1.0
+        self.freq: torch.Tensor | None = None
+        self.mult = 1.0
+
+    def frequencies(self) -> torch.Tensor:
+        i = torch.arange(self.dims // 2, dtype=torch.float64)
+        return self.base ** (-2.0 * i / max(self.dims, 1)) / self.factor
+
+    def finalize(self, device, dtype):
+        self.freq = self.frequencies().to(device)
+
+
+POSITION_ENCODINGS.register("half_rotary", HalfRotary)
 POSITION_ENCODINGS.register("rotary", RotaryEncoding)
 POSITION_ENCODINGS.register("scaled_rotary", ScaledRotary)
 POSITION_ENCODINGS.register("banded_rotary", BandedRotary)

@@ -147,7 +147,8 @@ def expected_tensors(model: Part) -> dict[str, tuple[tuple[int, ...], ParamSpec]
     for part in model.walk():
         for spec in part.param_specs().values():
             for src in spec.sources:
-                out[part.full_name(src.name)] = ((src.rows, *spec.shape[1:]), spec)
+                shape = (src.rows, *spec.shape[1:]) if spec.shape else ()   # (): one number
+                out[part.full_name(src.name)] = (shape, spec)
     return out
 
 
@@ -186,7 +187,7 @@ def load_weights(model: Part, source: TensorSource, device, dtype: torch.dtype,
             param = torch.zeros(spec.shape, dtype=target, device=device)
             for s in spec.sources:
                 tensor = source.get(part.full_name(s.name))
-                param[s.offset:s.offset + s.rows].copy_(tensor.to(device=device, dtype=target), non_blocking=False)
+                (param[s.offset:s.offset + s.rows] if spec.shape else param).copy_(tensor.to(device=device, dtype=target), non_blocking=False)
             part.params[local] = param
             done += 1
             if progress and done % 64 == 0:

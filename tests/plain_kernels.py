@@ -125,7 +125,106 @@ class PlainKernels:
         return silu_and_mul(self.linear(x, weight, bias, out_dtype=WIDE)).to(x.dtype)
 
     def materialize(self, x):
+        if hasattr(x, "terms"):    # a sum of scaled terms that a mixer handed on
+            out = torch.empty(tuple(x.shape), dtype=torch.float32)
+            return self.sum_norm(out, 0.0, x.terms, x.scales, None, 0.0, None)
         return x
+
+    # ---- the kernels of a stream that is normed after every sum, and of attention whose heads are worked together
+
+    def sum_norm(self, stream, alpha, summands, scales, weight, eps, out=None):
+        total = alpha * stream.to(WIDE) if alpha != 0 else torch.zeros(tuple(stream.shape), dtype=WIDE)
+        for y, s in zip(summands, scales):
+            total = total + s * y.to(WIDE)
+        if weight is not None:
+            total = total / torch.sqrt((total * total).mean(-1, keepdim=True) + eps) * weight.to(WIDE)
+        stream.copy_(total.to(stream.dtype))
+        if out is not None:
+            out.copy_(total.to(out.dtype))
+        return stream
+
+    def shift_rows(self, x, mu, out, state, state_off, cu_seqlens_q, slot_of_seq, token_seq):
+        width = x.shape[1]
+        out.zero_()
+        for b in range(slot_of_seq.numel()):
+            lo, hi, slot = int(cu_seqlens_q[b]), int(cu_seqlens_q[b + 1]), int(slot_of_seq[b])
+            if hi == lo or slot < 0:
+                continue
+            rows = x[lo:hi].to(WIDE)
+            kept = state[slot, state_off:state_off + width]
+            before = torch.cat((kept.to(WIDE)[None], rows[:-1]))
+            out[lo:hi] = (rows + (before - rows) * mu.to(WIDE)).to(out.dtype)
+            kept.copy_(rows[-1].to(kept.dtype))
+        return out
+
+    def qkv_rot_write(self, qkv, q_out, k_cache, v_cache, q_weight, k_weight, freq, rot_dims, positions, slots,
+                      num_heads, num_kv_heads, head_dim, value_dim, page_size, eps, v_source=None, v_blend=None,
+                      v_keep=None):
+        t = qkv.shape[0]
+        H, G, D, DV = num_heads, num_kv_heads, head_dim, value_dim
+        q, k, v = torch.split(qkv.to(WIDE)[:, :(H + G) * D + G * DV], [H * D, G * D, G * DV], dim=-1)
+        q, k = q.reshape(t, H, D), k.reshape(t, G, D)
+        if q_weight is not None:
+            q = q / torch.sqrt((q * q).mean(-1, keepdim=True) + eps) * q_weight.to(WIDE)
+        if k_weight is not None:
+            k = k / torch.sqrt((k * k).mean(-1, keepdim=True) + eps) * k_weight.to(WIDE)
+        if rot_dims:
+            half = rot_dims // 2
+            a = positions.to(WIDE)[:, None] * freq.to(WIDE)[None]
+            c, s = torch.cos(a)[:, None], torch.sin(a)[:, None]
+
+            def turn(x):
+                u, w = x[..., :half], x[..., half:rot_dims]
+                return torch.cat((u * c - w * s, w * c + u * s, x[..., rot_dims:]), -1)
+
+            q, k = turn(q), turn(k)
+        if v_keep is not None:
+            v_keep.copy_(v.to(v_keep.dtype))
+        if v_source is not None:
+            lam = v_blend.to(WIDE)
+            v = (1 - lam) * v + lam * v_source.to(WIDE)
+        v = v.reshape(t, G, DV)
+        q_out.copy_(q.to(q_out.dtype))
+        for i in range(t):
+            slot = int(slots[i])
+            if slot < 0:
+                continue
+            page, off = divmod(slot, page_size)
+            k_cache[page, :, off, :] = k[i].to(k_cache.dtype)
+            v_cache[page, :, :, off] = v[i].to(v_cache.dtype)
+        return q_out
+
+    def attention_together(self, q, k_cache, v_cache, out, token_seq, positions, block_tables, scale, head_scale=None,
+                           sink=None, talk=None, window=None, max_context_len=None):
+        tokens, H, D = q.shape
+        G, page_size = k_cache.shape[1], k_cache.shape[2]
+        for t in range(tokens):
+            seq = int(token_seq[t])
+            if seq < 0:
+                out[t] = 0
+                continue
+            pos = int(positions[t])
+            first = max(0, pos - window + 1) if window else 0
+            keys = torch.arange(first, pos + 1)
+            pages = block_tables[seq].long()[keys // page_size]
+            offs = keys % page_size
+            k = k_cache[pages, :, offs, :].to(WIDE).repeat_interleave(H // G, dim=1)     # [n, H, D]
+            v = v_cache[pages, :, :, offs].to(WIDE).repeat_interleave(H // G, dim=1)     # [n, H, DV]
+            s = torch.einsum("hd,nhd->hn", q[t].to(WIDE), k) * scale
+            if head_scale is not None:
+                s = s * head_scale.to(WIDE)[:, None]
+            m = s.max(-1, keepdim=True).values
+            if sink is not None:
+                m = torch.maximum(m, sink.to(WIDE)[:, None])
+            e = torch.exp(s - m)
+            den = e.sum(-1, keepdim=True)
+            if sink is not None:
+                den = den + torch.exp(sink.to(WIDE)[:, None] - m)
+            w = e / den
+            if talk is not None:
+                w = talk.to(WIDE) @ w
+            out[t] = torch.einsum("hn,nhd->hd", w, v).to(out.dtype)
+        return out
 
     # ---- the kernels of the layer-norm / latent-attention / delta-rule / routed-experts parts
 
