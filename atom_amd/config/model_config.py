@@ -657,9 +657,9 @@ class SavidraConfig(ModelConfig):
             if kind == "attention":
                 attention(m, mw)
                 if m.get("v_mix"):
-                    size = m["kv_heads"] * m["vdim"]
+                    size = (m["kv_heads"], m["vdim"])
                     if mixed_values is not None and size != mixed_values:
-                        raise ConfigError(f"{where}: layers that blend their values need values of one size")
+                        raise ConfigError(f"{where}: layers that blend their values need value heads of one number and size")
                     mixed_values = size
             else:
                 attention(_need(m, "left", dict, mw), f"{mw}'s left")

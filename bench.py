@@ -331,6 +331,40 @@ def leduvik_pair(size: str) -> tuple[dict, dict]:
     return ledu, qwen
 
 
+# The Savidra side has four layers (attention side by side with the delta rule twice, attention with a sink and blended
+# values twice), each with a ReLU-gated feed-forward, token shift before every mixer and a norm after every sum; the
+# Qwen3 side four layers of the same width with a gated feed-forward of the same size.
+
+def savidra_pair(size: str) -> tuple[dict, dict]:
+    width, heads, ff, vocab = {
+        "1k": (1024, 8, 2816, 32768),
+        "2k": (2048, 16, 5632, 32768),
+        "4k": (4096, 32, 11264, 65536),
+    }[size]
+    kv = max(1, heads // 4)
+    attn = {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "v_mix": True,
+            "rot": {"base": 1000000.0, "dims": 64}}
+    left = {"heads": heads // 2, "kv_heads": max(1, kv // 2), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "conv": 3,
+            "rot": {"base": 500000.0, "dims": 128, "scaling": {"factor": 8.0}}}
+    right = {"heads": heads // 2, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "conv": 4, "decay_rank": 64,
+             "gate_rank": 64}
+    side = {"left": left, "right": right, "left_scale": 0.6, "right_scale": 1.1}
+    dense = {"kind": "dense", "ff": ff}
+    savi = {"architecture": "Savidra", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "postln_alpha": 2.0,
+            "layers": [{"type": "parallel", "mixer": side, "mlp": dense},
+                       {"type": "attention", "mixer": attn, "mlp": dense},
+                       {"type": "parallel", "mixer": side, "mlp": dense},
+                       {"type": "attention", "mixer": attn, "mlp": dense}]}
+    qwen = dict(QWEN3_8B, num_hidden_layers=4, hidden_size=width, num_attention_heads=heads,
+                num_key_value_heads=kv, intermediate_size=ff, vocab_size=vocab)
+    return savi, qwen
+
+
+def run_savidra(args) -> dict:
+    """Prefill and decode throughput of Savidra and of Qwen3 at equal size, one engine after the other."""
+    return run_design(args, "savidra", "Savidra", savidra_pair, args.savidra)
+
+
 def run_lotorax(args) -> dict:
     """Prefill and decode throughput of Lotorax and of Qwen3 at equal size, one engine after the other."""
     return run_design(args, "lotorax", "Lotorax", lotorax_pair, args.lotorax)
@@ -645,6 +679,9 @@ def main() -> int:
     ap.add_argument("--leduvik", type=str, default="", metavar="SIZE[,SIZE]",
                     help="the Leduvik design beside Qwen3 at equal size (1k, 2k, 4k: the width): prefill of --context "
                          "tokens and decode at --batch, four layers each")
+    ap.add_argument("--savidra", type=str, default="", metavar="SIZE[,SIZE]",
+                    help="the Savidra design beside Qwen3 at equal size (1k, 2k, 4k: the width): prefill of --context "
+                         "tokens and decode at --batch, four layers each")
     ap.add_argument("--budget", type=int, default=None,
                     help="the scheduler's token budget of a step (mixed: 512 + N by default, so that portions stay 512)")
     ap.add_argument("--temperature", type=float, default=0.0, help="of the decode steps' sampling (0: greedy)")
@@ -675,6 +712,9 @@ def main() -> int:
         return 0
     if args.leduvik:
         print(json.dumps(run_leduvik(args)), flush=True)
+        return 0
+    if args.savidra:
+        print(json.dumps(run_savidra(args)), flush=True)
         return 0
     args.shape = args.shape or "8b"
     line = run_shape(args)

@@ -60,7 +60,7 @@ SAVI_A = {
         {"type": "attention", "mixer": _attn(4, 2, 10, 6, 0.4, _rot(6, 1000.0), v_mix=True), "mlp": _dense(56)},
         {"type": "parallel", "mixer": _side(_attn(6, 3, 6, 4, 0.5, _rot(6, 300.0, 4.0), conv=2), _delta(4, 2, 5, 7, 3),
                                             0.7, 1.2), "mlp": None},
-        {"type": "attention", "mixer": _attn(2, 1, 12, 12, 0.3, _rot(4, 50.0), v_mix=True), "mlp": _dense(48)},
+        {"type": "attention", "mixer": _attn(2, 2, 12, 6, 0.3, _rot(4, 50.0), v_mix=True), "mlp": _dense(48)},
         {"type": "attention", "mixer": _attn(3, 3, 8, 5, 0.35, _rot(8, 10000.0), v_mix=False), "mlp": _dense(32)},
     ],
 }
