@@ -12,6 +12,10 @@
 // values.  Keys are taken 64 at a time in chunks counted from position 0, so a token's result depends on its own
 // keys only: not on the batch, not on how a prompt was cut, not on which pages hold the keys.
 //
+// Few tokens with long contexts (decode steps) are cut over `parts` blocks a (token, head set): every part takes a run
+// of whole chunks.  One launch leaves each part's maximum and sum, a second merges them (a few numbers), forms the
+// weights of its own keys and leaves its share of the weighted sum, which a third adds up in the order of the parts.
+//
 // Pages: keys [pages, G, page, D]; values [pages, G, DV, page].
 #include "common.h"
 
@@ -24,7 +28,49 @@ struct TogetherArgs {
   int H, G, D, DV, page_size, window;
   float scale;
   const float* head_scale; const float* sink; const float* talk;
+  int parts;          // > 1: the keys of a token are cut over this many blocks
+  float* ws_ml;       // [tokens, H, parts, 2]: a part's maximum and sum
+  float* ws_o;        // [tokens, parts, H, DV]: a part's share of the weighted sum
 };
+
+// The chunks [c0, c1) of a token's visible keys that part `part` takes, counted from the chunk that holds `first`.
+__device__ __forceinline__ void together_part(int start, int pos, int parts, int part, int& base0, int& base1) {
+  const int chunks = (pos - start) / kTogetherChunk + 1;
+  const int each = (chunks + parts - 1) / parts;
+  const int c0 = part * each, c1 = c0 + each < chunks ? c0 + each : chunks;
+  base0 = start + c0 * kTogetherChunk;
+  base1 = start + c1 * kTogetherChunk;     // exclusive; base0 >= base1: the part is empty
+}
+
+// q . k over D entries; 16 bytes of the key row a load where `wide` says the rows allow it
+__device__ __forceinline__ float together_dot(const float* __restrict__ qr, const float* __restrict__ kr, int D, bool wide) {
+  float d = 0.f;
+  if (wide) {
+    for (int i = 0; i < D; i += 4) {
+      const float4 k4 = *reinterpret_cast<const float4*>(kr + i);
+      d += qr[i] * k4.x + qr[i + 1] * k4.y + qr[i + 2] * k4.z + qr[i + 3] * k4.w;
+    }
+  } else {
+    for (int i = 0; i < D; ++i) d += qr[i] * kr[i];
+  }
+  return d;
+}
+
+__device__ __forceinline__ float together_dot(const float* __restrict__ qr, const bf16_t* __restrict__ kr, int D, bool wide) {
+  float d = 0.f;
+  if (wide) {
+    union Pack { uint4 raw; bf16_t e[8]; };
+    for (int i = 0; i < D; i += 8) {
+      Pack p;
+      p.raw = *reinterpret_cast<const uint4*>(kr + i);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) d += qr[i + e] * to_f32(p.e[e]);
+    }
+  } else {
+    for (int i = 0; i < D; ++i) d += qr[i] * to_f32(kr[i]);
+  }
+  return d;
+}
 
 // scores of the block's heads against the keys lo .. hi of a chunk that starts at base, into s[hb][kTogetherChunk]
 // (-inf outside lo .. hi)
@@ -40,9 +86,7 @@ __device__ __forceinline__ void together_scores(const TogetherArgs& a, const T* 
       const int h = h0 + hh;
       const int page = table[key / a.page_size], off = key % a.page_size;
       const T* kr = k_cache + (((size_t)page * a.G + h / group) * a.page_size + off) * (size_t)a.D;
-      const float* qr = qs + (size_t)hh * a.D;
-      float d = 0.f;
-      for (int i = 0; i < a.D; ++i) d += qr[i] * to_f32(kr[i]);
+      const float d = together_dot(qs + (size_t)hh * a.D, kr, a.D, a.D % (16 / (int)sizeof(T)) == 0);
       v = d * a.scale * (a.head_scale != nullptr ? a.head_scale[h] : 1.f);
     }
     s[item] = v;
@@ -165,6 +209,146 @@ attention_together_kernel(const T* __restrict__ q, const T* __restrict__ k_cache
   }
 }
 
+// PASS 1: the maximum and sum of every head over this part's keys.  PASS 2: the parts' maxima and sums merged, then
+// this part's weights, their mixing and its share of the weighted sum.
+template <typename T, int PASS>
+__global__ void __launch_bounds__(kTogetherThreads)
+attention_together_part_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                               TogetherArgs a) {
+  extern __shared__ float lds[];
+  const int t = blockIdx.x, part = blockIdx.z;
+  const int HB = a.talk != nullptr ? a.H : a.H / a.G;
+  const int h0 = a.talk != nullptr ? 0 : blockIdx.y * HB;
+  float* qs = lds;
+  float* s = qs + (size_t)HB * a.D;
+  float* mixed = s + (size_t)HB * kTogetherChunk;
+  float* top = mixed + (a.talk != nullptr ? (size_t)HB * kTogetherChunk : 0);
+  float* den = top + HB;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1), wave = tid / kWave;
+  constexpr int waves = kTogetherThreads / kWave;
+  const int seq = a.token_seq[t];
+  const int items = HB * a.DV;
+  if (seq < 0) {   // padding row: no maximum, no sum, no share
+    if (PASS == 1) {
+      for (int hh = tid; hh < HB; hh += kTogetherThreads) {
+        float* ml = a.ws_ml + (((size_t)t * a.H + h0 + hh) * a.parts + part) * 2;
+        ml[0] = -INFINITY, ml[1] = 0.f;
+      }
+    } else {
+      for (int e = tid; e < items; e += kTogetherThreads) a.ws_o[(((size_t)t * a.parts + part) * a.H + h0) * a.DV + e] = 0.f;
+    }
+    return;
+  }
+  const int pos = a.positions[t];
+  const int* table = a.block_tables + (size_t)seq * a.max_blocks;
+  for (int e = tid; e < HB * a.D; e += kTogetherThreads) qs[e] = to_f32(q[((size_t)t * a.H + h0) * a.D + e]);
+  const int first = (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
+  const int start = first / kTogetherChunk * kTogetherChunk;
+  int base0, base1;
+  together_part(start, pos, a.parts, part, base0, base1);
+  if (PASS == 1) {
+    for (int e = tid; e < HB; e += kTogetherThreads) top[e] = -INFINITY, den[e] = 0.f;
+    __syncthreads();
+    for (int base = base0; base < base1; base += kTogetherChunk) {
+      const int lo = base > first ? base : first;
+      const int hi = base + kTogetherChunk - 1 < pos ? base + kTogetherChunk - 1 : pos;
+      together_scores(a, k_cache, table, qs, s, h0, HB, base, lo, hi);
+      __syncthreads();
+      for (int hh = wave; hh < HB; hh += waves) {
+        const float v = s[hh * kTogetherChunk + lane];
+        const float m_old = top[hh];
+        const float m_new = fmaxf(m_old, wave_max(v));
+        const float sum = wave_sum(expf(v - m_new));
+        if (lane == 0) {
+          den[hh] = den[hh] * (m_old == -INFINITY ? 0.f : expf(m_old - m_new)) + sum;
+          top[hh] = m_new;
+        }
+      }
+      __syncthreads();
+    }
+    for (int hh = tid; hh < HB; hh += kTogetherThreads) {
+      float* ml = a.ws_ml + (((size_t)t * a.H + h0 + hh) * a.parts + part) * 2;
+      ml[0] = top[hh], ml[1] = den[hh];
+    }
+    return;
+  }
+  // the parts' maxima and sums, in the order of the parts
+  for (int hh = tid; hh < HB; hh += kTogetherThreads) {
+    const float* ml = a.ws_ml + ((size_t)t * a.H + h0 + hh) * a.parts * 2;
+    float m = a.sink != nullptr ? a.sink[h0 + hh] : -INFINITY;
+    for (int p = 0; p < a.parts; ++p) m = fmaxf(m, ml[2 * p]);
+    float l = a.sink != nullptr ? expf(a.sink[h0 + hh] - m) : 0.f;
+    for (int p = 0; p < a.parts; ++p)
+      if (ml[2 * p] != -INFINITY) l += ml[2 * p + 1] * expf(ml[2 * p] - m);
+    top[hh] = m;
+    den[hh] = 1.f / l;
+  }
+  __syncthreads();
+  float acc[kTogetherAcc];
+#pragma unroll
+  for (int r = 0; r < kTogetherAcc; ++r) acc[r] = 0.f;
+  const int group = a.H / a.G;
+  for (int base = base0; base < base1; base += kTogetherChunk) {
+    const int lo = base > first ? base : first;
+    const int hi = base + kTogetherChunk - 1 < pos ? base + kTogetherChunk - 1 : pos;
+    together_scores(a, k_cache, table, qs, s, h0, HB, base, lo, hi);
+    for (int item = tid; item < HB * kTogetherChunk; item += kTogetherThreads) {
+      const int hh = item / kTogetherChunk;
+      s[item] = expf(s[item] - top[hh]) * den[hh];
+    }
+    __syncthreads();
+    const float* w = s;
+    if (a.talk != nullptr) {
+      for (int item = tid; item < HB * kTogetherChunk; item += kTogetherThreads) {
+        const int hh = item / kTogetherChunk, j = item - hh * kTogetherChunk;
+        const float* row = a.talk + (size_t)hh * a.H;
+        float m = 0.f;
+        for (int g = 0; g < a.H; ++g) m += row[g] * s[g * kTogetherChunk + j];
+        mixed[item] = m;
+      }
+      __syncthreads();
+      w = mixed;
+    }
+#pragma unroll
+    for (int r = 0; r < kTogetherAcc; ++r) {
+      const int e = tid + r * kTogetherThreads;
+      if (e < items) {
+        const int hh = e / a.DV, i = e - hh * a.DV;
+        const int kvh = (h0 + hh) / group;
+        const float* wr = w + hh * kTogetherChunk - base;
+        float sum = acc[r];
+        for (int key = lo; key <= hi;) {
+          const int page = table[key / a.page_size], off = key % a.page_size;
+          int run = a.page_size - off;
+          if (run > hi - key + 1) run = hi - key + 1;
+          const T* vr = v_cache + (((size_t)page * a.G + kvh) * a.DV + i) * (size_t)a.page_size + off;
+          for (int u = 0; u < run; ++u) sum += wr[key + u] * to_f32(vr[u]);
+          key += run;
+        }
+        acc[r] = sum;
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int r = 0; r < kTogetherAcc; ++r) {
+    const int e = tid + r * kTogetherThreads;
+    if (e < items) a.ws_o[(((size_t)t * a.parts + part) * a.H + h0) * a.DV + e] = acc[r];
+  }
+}
+
+template <typename T>
+__global__ void together_sum_parts_kernel(const float* __restrict__ ws_o, T* __restrict__ out, int parts, int row, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t t = idx / row;
+  const size_t e = idx - t * row;
+  float sum = 0.f;
+  for (int p = 0; p < parts; ++p) sum += ws_o[(t * parts + p) * row + e];
+  out[idx] = from_f32<T>(sum);
+}
+
 static size_t together_lds(int H, int G, int D, bool talk) {
   const int HB = talk ? H : H / G;
   return ((size_t)HB * D + (size_t)HB * kTogetherChunk * (talk ? 2 : 1) + 2 * (size_t)HB) * sizeof(float);
@@ -174,7 +358,7 @@ ATOM_EXPORT int atom_attention_together(const void* q, const void* k_cache, cons
                                         const int* token_seq, const int* positions, const int* block_tables,
                                         int max_blocks, int tokens, int H, int G, int D, int DV, int page_size,
                                         float scale, const float* head_scale, const float* sink, const float* talk,
-                                        int window, hipStream_t stream) {
+                                        int window, int parts, float* ws_ml, float* ws_o, hipStream_t stream) {
   if (tokens < 0 || H <= 0 || G <= 0 || D <= 0 || DV <= 0 || page_size <= 0 || max_blocks <= 0) return ATOM_BAD_SHAPE;
   if (H % G || window < 0) return ATOM_BAD_SHAPE;
   if (q == nullptr || k_cache == nullptr || v_cache == nullptr || out == nullptr) return ATOM_BAD_SHAPE;
@@ -185,9 +369,25 @@ ATOM_EXPORT int atom_attention_together(const void* q, const void* k_cache, cons
   const size_t smem = together_lds(H, G, D, mixes);
   if (smem > 64 * 1024) return ATOM_TOO_LARGE;
   if (tokens == 0) return ATOM_OK;
-  TogetherArgs a{token_seq, positions, block_tables, max_blocks, H, G, D, DV, page_size, window, scale, head_scale, sink, talk};
-  dim3 grid(tokens, mixes ? 1 : G), block(kTogetherThreads);
-  ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((attention_together_kernel<T>), grid, block, smem, stream, (const T*)q,
-                                                 (const T*)k_cache, (const T*)v_cache, (T*)out, a));
+  if (parts < 1 || parts > 65535 || (parts > 1 && (ws_ml == nullptr || ws_o == nullptr))) return ATOM_BAD_SHAPE;
+  TogetherArgs a{token_seq, positions, block_tables, max_blocks, H, G, D, DV, page_size, window, scale, head_scale, sink,
+                 talk, parts, ws_ml, ws_o};
+  dim3 grid(tokens, mixes ? 1 : G, parts), block(kTogetherThreads);
+  if (parts == 1) {
+    ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((attention_together_kernel<T>), grid, block, smem, stream, (const T*)q,
+                                                   (const T*)k_cache, (const T*)v_cache, (T*)out, a));
+    return launch_status();
+  }
+  const size_t total = (size_t)tokens * H * DV;
+  const size_t blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffffu) return ATOM_TOO_LARGE;
+  ATOM_DISPATCH_DTYPE(dtype, {
+    hipLaunchKernelGGL((attention_together_part_kernel<T, 1>), grid, block, smem, stream, (const T*)q, (const T*)k_cache,
+                       (const T*)v_cache, a);
+    hipLaunchKernelGGL((attention_together_part_kernel<T, 2>), grid, block, smem, stream, (const T*)q, (const T*)k_cache,
+                       (const T*)v_cache, a);
+    hipLaunchKernelGGL((together_sum_parts_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream, ws_o, (T*)out, parts,
+                       H * DV, total);
+  });
   return launch_status();
 }

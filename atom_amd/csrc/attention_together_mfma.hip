@@ -1,0 +1,255 @@
+// Attention with a token's heads worked through together (see attention_together.hip for what is computed), on the
+// matrix cores: bfloat16, key heads of 64 or 128 entries, value heads of 32, 64 or 128, up to 16 heads a block,
+// pages of a multiple of four tokens.  For steps that bring prompt portions.
+//
+// A block of four waves owns a tile of up to 16 consecutive query tokens of one request and a set of heads: all of
+// them when the heads' weights are mixed, else the query heads of one key/value head.  The heads are dealt out to the
+// waves.  Both products are formed transposed, so a lane always holds values of one query token (lane % 16):
+//
+//     S^T[key][query] = K[key][:] . Q[query][:]        A = K rows from the key pages, B = Q (kept in registers)
+//     O^T[d][query]   = V^T[d][key] . W[query][key]    A = V^T rows (value pages hold keys contiguously), B = W
+//
+// The first product leaves lane (query, g = lane / 16) with the scores of keys 4g .. 4g + 3 of a chunk of 16, which
+// is the B operand of the second.  The keys are walked twice: once for every (query, head)'s maximum and sum, which
+// are per-lane numbers, then for the finished weights.  Mixing the heads is entrywise in this layout: the waves
+// exchange their heads' weights of a chunk through LDS (two buffers in turn, one barrier a chunk) and every wave
+// forms sum_g talk[h, g] w_g for its own heads.  Chunks are counted from position 0.
+//
+// A block finds its request and tile from the block index alone: tile j of request s has the place
+// cu[s] / 16 + s + j, which is unique, so the launch needs no list of tiles from the host.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(4))) float tg_f32x4;
+typedef __attribute__((ext_vector_type(4))) short tg_s16x4;
+typedef __attribute__((ext_vector_type(8))) __bf16 tg_bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 tg_bf16x4;
+
+constexpr int kTileWaves = 4;
+constexpr int kTileRows = 16;
+
+struct TogetherTileArgs {
+  const bf16_t* q; const bf16_t* k_cache; const bf16_t* v_cache; bf16_t* out;
+  const int* cu_q; const int* positions; const int* block_tables;
+  int max_blocks, num_seqs, H, G, page_size, window;
+  float scale_log2;
+  const float* head_scale; const float* sink; const float* talk;
+};
+
+template <int D, int NDV, int HPW>
+__global__ void __launch_bounds__(kTileWaves * kWave)
+together_tile_kernel(TogetherTileArgs a) {
+  constexpr int DV = 16 * NDV;
+  constexpr float kLog2e = 1.4426950408889634f;
+  __shared__ tg_f32x4 pbuf[2][HPW * kTileWaves][kWave];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int n = lane & 15, g4 = lane >> 4;
+  // the request and the tile of this block: the last s with cu[s] / 16 + s <= b
+  const int b = blockIdx.x;
+  int lo = 0, hi = a.num_seqs - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (a.cu_q[mid] / kTileRows + mid <= b) lo = mid; else hi = mid - 1;
+  }
+  const int seq = lo;
+  const int t_begin = a.cu_q[seq], t_end = a.cu_q[seq + 1];
+  const int tile = b - (t_begin / kTileRows + seq);
+  if (tile < 0 || tile * kTileRows >= t_end - t_begin) return;   // the whole block leaves together
+  const int t0 = t_begin + tile * kTileRows;
+  const int rows = t_end - t0 < kTileRows ? t_end - t0 : kTileRows;
+  const bool row_ok = n < rows;
+  const int pos = row_ok ? a.positions[t0 + n] : -1;
+  const int pos_lo = a.positions[t0], pos_hi = a.positions[t0 + rows - 1];
+  const int first_row = (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
+  const int first_blk = (a.window > 0 && pos_lo - a.window + 1 > 0) ? pos_lo - a.window + 1 : 0;
+  const int* table = a.block_tables + (size_t)seq * a.max_blocks;
+  const bool mixes = a.talk != nullptr;
+  const int HB = mixes ? a.H : a.H / a.G;
+  const int h0 = mixes ? 0 : blockIdx.y * HB;
+  const int group = a.H / a.G;
+  const int ps = a.page_size;
+
+  tg_bf16x8 qf[HPW][D / 32];
+  float top[HPW], den[HPW], hs[HPW];
+  bool own[HPW];
+#pragma unroll
+  for (int u = 0; u < HPW; ++u) {
+    const int hh = wave + kTileWaves * u;
+    own[u] = hh < HB;
+    const int h = h0 + (own[u] ? hh : 0);
+    const bf16_t* qr = a.q + ((size_t)(t0 + (row_ok ? n : 0)) * a.H + h) * D + 8 * g4;
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j) {
+      tg_bf16x8 v = *reinterpret_cast<const tg_bf16x8*>(qr + 32 * j);
+      if (!row_ok || !own[u]) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = (__bf16)0.f;
+      }
+      qf[u][j] = v;
+    }
+    top[u] = -INFINITY;
+    den[u] = 0.f;
+    hs[u] = a.scale_log2 * (a.head_scale != nullptr ? a.head_scale[h] : 1.f);
+  }
+
+  // scores of head u against the 16 keys from base, in the exp2 domain, -inf where the lane's query does not see the key
+  auto scores = [&](int u, int base) -> tg_f32x4 {
+    const int h = h0 + wave + kTileWaves * u;
+    int key = base + n;                       // the key row this lane brings to the A operand
+    if (key > pos_hi) key = pos_hi;           // beyond the tile's last key: any valid row, masked below
+    const int page = table[key / ps], off = key - key / ps * ps;
+    const bf16_t* kr = a.k_cache + (((size_t)page * a.G + h / group) * ps + off) * (size_t)D + 8 * g4;
+    tg_f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j)
+      s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const tg_bf16x8*>(kr + 32 * j), qf[u][j], s, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int k = base + 4 * g4 + i;
+      s[i] = (k >= first_row && k <= pos) ? s[i] * hs[u] : -INFINITY;
+    }
+    return s;
+  };
+
+  const int start = first_blk / kTileRows * kTileRows;
+  // every (query, head)'s maximum and sum
+  for (int base = start; base <= pos_hi; base += kTileRows) {
+#pragma unroll
+    for (int u = 0; u < HPW; ++u) {
+      if (!own[u]) continue;
+      const tg_f32x4 s = scores(u, base);
+      const float cm = rows_max(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
+      const float m_new = fmaxf(top[u], cm);
+      // no branch around the exchange between lanes: a query that has seen no key yet keeps a sum of zero
+      const float m_at = m_new == -INFINITY ? 0.f : m_new;
+      const float part = exp2f(s[0] - m_at) + exp2f(s[1] - m_at) + exp2f(s[2] - m_at) + exp2f(s[3] - m_at);
+      den[u] = den[u] * exp2f(top[u] - m_at) + rows_sum(part);
+      top[u] = m_new;
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < HPW; ++u) {
+    if (!own[u]) continue;
+    float m = top[u], l = den[u];
+    if (a.sink != nullptr && row_ok) {
+      const float sk = a.sink[h0 + wave + kTileWaves * u] * kLog2e;
+      const float m_new = fmaxf(m, sk);
+      l = l * exp2f(m - m_new) + exp2f(sk - m_new);
+      m = m_new;
+    }
+    den[u] = l > 0.f ? 1.f / l : 0.f;
+    top[u] = m == -INFINITY ? 0.f : m;
+  }
+
+  // the weights, their mixing, the weighted sum of the values
+  tg_f32x4 acc[HPW][NDV];
+#pragma unroll
+  for (int u = 0; u < HPW; ++u)
+#pragma unroll
+    for (int t = 0; t < NDV; ++t) acc[u][t] = tg_f32x4{0.f, 0.f, 0.f, 0.f};
+  int turn = 0;
+  for (int base = start; base <= pos_hi; base += kTileRows, turn ^= 1) {
+    tg_f32x4 w[HPW];
+#pragma unroll
+    for (int u = 0; u < HPW; ++u) {
+      w[u] = tg_f32x4{0.f, 0.f, 0.f, 0.f};
+      if (!own[u]) continue;
+      const tg_f32x4 s = scores(u, base);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w[u][i] = exp2f(s[i] - top[u]) * den[u];   // exp2(-inf) = 0 where unseen
+      if (mixes) pbuf[turn][wave + kTileWaves * u][lane] = w[u];
+    }
+    if (mixes) {
+      __syncthreads();
+#pragma unroll
+      for (int u = 0; u < HPW; ++u) {
+        if (!own[u]) continue;
+        const float* row = a.talk + (size_t)(wave + kTileWaves * u) * a.H;
+        tg_f32x4 m = {0.f, 0.f, 0.f, 0.f};
+        for (int g = 0; g < a.H; ++g) {
+          const float c = row[g];
+          const tg_f32x4 p = pbuf[turn][g][lane];
+          m[0] += c * p[0], m[1] += c * p[1], m[2] += c * p[2], m[3] += c * p[3];
+        }
+        w[u] = m;
+      }
+    }
+    // the four keys this lane brings to the A operand of the second product: one page holds them
+    int key0 = base + 4 * g4;
+    if (key0 > pos_hi) key0 = pos_hi & ~3;      // unseen by every query: any valid place, the weights are zero
+    const int page = table[key0 / ps], off = key0 - key0 / ps * ps;
+#pragma unroll
+    for (int u = 0; u < HPW; ++u) {
+      if (!own[u]) continue;
+      const int kvh = (h0 + wave + kTileWaves * u) / group;
+      tg_bf16x4 pb;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) pb[i] = (__bf16)w[u][i];
+      const bf16_t* vr = a.v_cache + (((size_t)page * a.G + kvh) * DV + n) * (size_t)ps + off;
+#pragma unroll
+      for (int t = 0; t < NDV; ++t) {
+        const tg_bf16x4 vf = *reinterpret_cast<const tg_bf16x4*>(vr + (size_t)16 * t * ps);
+        acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(tg_s16x4, vf),
+                                                              __builtin_bit_cast(tg_s16x4, pb), acc[u][t], 0, 0, 0);
+      }
+    }
+  }
+  if (!row_ok) return;
+#pragma unroll
+  for (int u = 0; u < HPW; ++u) {
+    if (!own[u]) continue;
+    bf16_t* dst = a.out + ((size_t)(t0 + n) * a.H + h0 + wave + kTileWaves * u) * DV + 4 * g4;
+#pragma unroll
+    for (int t = 0; t < NDV; ++t) {
+      tg_bf16x4 o;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] = (__bf16)acc[u][t][i];
+      *reinterpret_cast<tg_bf16x4*>(dst + 16 * t) = o;
+    }
+  }
+}
+
+static bool together_tile_takes(int H, int G, int D, int DV, int page_size, bool mixes) {
+  const int HB = mixes ? H : H / G;
+  return (D == 64 || D == 128) && (DV == 32 || DV == 64 || DV == 128) && HB >= 1 && HB <= 16 && page_size % 4 == 0;
+}
+
+ATOM_EXPORT int atom_attention_together_tiles_supports(int H, int G, int D, int DV, int page_size, int mixes) {
+  return (H > 0 && G > 0 && H % G == 0 && together_tile_takes(H, G, D, DV, page_size, mixes != 0)) ? 1 : 0;
+}
+
+template <int D, int NDV>
+static int together_tile_launch(const TogetherTileArgs& a, dim3 grid, int HB, hipStream_t stream) {
+  const dim3 block(kTileWaves * kWave);
+  if (HB <= 4) hipLaunchKernelGGL((together_tile_kernel<D, NDV, 1>), grid, block, 0, stream, a);
+  else if (HB <= 8) hipLaunchKernelGGL((together_tile_kernel<D, NDV, 2>), grid, block, 0, stream, a);
+  else hipLaunchKernelGGL((together_tile_kernel<D, NDV, 4>), grid, block, 0, stream, a);
+  return launch_status();
+}
+
+ATOM_EXPORT int atom_attention_together_tiles(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                              const int* cu_q, const int* positions, const int* block_tables,
+                                              int max_blocks, int tokens, int num_seqs, int H, int G, int D, int DV,
+                                              int page_size, float scale, const float* head_scale, const float* sink,
+                                              const float* talk, int window, hipStream_t stream) {
+  if (tokens < 0 || num_seqs <= 0 || H <= 0 || G <= 0 || H % G || max_blocks <= 0 || window < 0) return ATOM_BAD_SHAPE;
+  if (q == nullptr || k_cache == nullptr || v_cache == nullptr || out == nullptr) return ATOM_BAD_SHAPE;
+  if (cu_q == nullptr || positions == nullptr || block_tables == nullptr) return ATOM_BAD_SHAPE;
+  const bool mixes = talk != nullptr;
+  if (!together_tile_takes(H, G, D, DV, page_size, mixes)) return ATOM_UNSUPPORTED;
+  if (tokens == 0) return ATOM_OK;
+  const int HB = mixes ? H : H / G;
+  TogetherTileArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, cu_q, positions,
+                     block_tables, max_blocks, num_seqs, H, G, page_size, window, scale * 1.4426950408889634f,
+                     head_scale, sink, talk};
+  const dim3 grid(tokens / kTileRows + num_seqs + 1, mixes ? 1 : G);
+#define ATOM_TILE(DD, NN) return together_tile_launch<DD, NN>(a, grid, HB, stream)
+  if (D == 64) {
+    if (DV == 32) ATOM_TILE(64, 2);
+    if (DV == 64) ATOM_TILE(64, 4);
+    ATOM_TILE(64, 8);
+  }
+  if (DV == 32) ATOM_TILE(128, 2);
+  if (DV == 64) ATOM_TILE(128, 4);
+  ATOM_TILE(128, 8);
+#undef ATOM_TILE
+}

@@ -199,7 +199,7 @@ class HipKernels:
                    "atom_step_decay", "atom_group_norm_gate", "atom_qkv_plain_write", "atom_narrow_heads",
                    "atom_mean_of_norms", "atom_embedding_positions", "atom_unary_act", "atom_stream_add", "atom_scale_rows",
                    "atom_stream_norm", "atom_sum_norm", "atom_shift_rows", "atom_qkv_rot_write",
-                   "atom_attention_together"):
+                   "atom_attention_together", "atom_attention_together_tiles", "atom_attention_together_tiles_supports"):
             getattr(self.lib, fn).restype = ctypes.c_int
         self.allow_library_gemm = True
         # bfloat16 products of few rows run this library's own weight-streaming kernels: up to 64 rows, and
@@ -223,6 +223,7 @@ class HipKernels:
         self.prefill_key_halves = None
         self.prefill_low_blocks = None   # True / False forces 16 / 32 tokens a wave in the blocks of eight waves
         self.use_fused_decode = True    # decode-only steps of few rows: norm, rotation and cache write inside attention
+        self.use_together_tiles = True  # attention with the heads together on the matrix cores, for prompt portions
         self.use_mfma_latent = True     # attention over latent pages on the matrix cores (bfloat16, sizes it is built for)
         # routed experts: from this many (token, choice) pairs on, the pairs are sorted by expert and run as grouped
         # products on the matrix cores; below, every pair reads its expert's rows itself
@@ -1691,12 +1692,17 @@ class HipKernels:
 
     def attention_together(self, q, k_cache, v_cache, out, token_seq, positions, block_tables, scale: float,
                            head_scale=None, sink=None, talk=None, window: int | None = None,
-                           max_context_len: int | None = None):
+                           max_context_len: int | None = None, cu_seqlens_q=None, max_q_len: int | None = None,
+                           parts: int | None = None):
         """Softmax attention of the step's queries over the pages with a token's heads worked through together:
         ``head_scale`` (float32 [H]) multiplies the scaled scores of a head, ``sink`` (float32 [H]) joins the
         softmax's denominator as ``exp(sink[h])`` without a value, ``talk`` (float32 [H, H]) mixes the heads'
         finished weights, ``w_h <- sum_g talk[h, g] w_g``, before head h applies them to the values of its own
-        key/value head.  Value heads [pages, G, DV, page] may differ in size from key heads [pages, G, page, D]."""
+        key/value head.  Value heads [pages, G, DV, page] may differ in size from key heads [pages, G, page, D].
+
+        A step with prompt portions (``max_q_len`` > 1, ``cu_seqlens_q`` given) runs on the matrix cores where the
+        sizes allow (bfloat16; tiles of 16 tokens of a request); otherwise a block a (token, set of heads), with the
+        keys of few tokens cut over ``parts`` blocks (None: chosen so that the launch fills the chip)."""
         tokens, H, D = q.shape
         _, G, page_size, _ = k_cache.shape
         DV = v_cache.shape[2]
@@ -1715,10 +1721,32 @@ class HipKernels:
                 self._check(name, w, torch.float32, (H,))
         if talk is not None:
             self._check("head mixing", talk, torch.float32, (H, H))
+        if (self.use_together_tiles and dt == torch.bfloat16 and cu_seqlens_q is not None and (max_q_len or 0) > 1
+                and self.lib.atom_attention_together_tiles_supports(H, G, D, DV, page_size, int(talk is not None))):
+            seqs = cu_seqlens_q.numel() - 1
+            self._check("cu_seqlens_q", cu_seqlens_q, torch.int32, (seqs + 1,))
+            if block_tables.shape[0] != seqs:
+                raise KernelError("attention: one block table row per request is needed")
+            self._done("attention_together_tiles", self.lib.atom_attention_together_tiles(
+                _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(cu_seqlens_q), _ptr(positions), _ptr(block_tables),
+                block_tables.shape[1], tokens, seqs, H, G, D, DV, page_size, ctypes.c_float(scale), _ptr(head_scale),
+                _ptr(sink), _ptr(talk), int(window or 0), self._stream()))
+            return out
+        sets = tokens * (1 if talk is not None else G)
+        if parts is None:
+            reach = block_tables.shape[1] * page_size if max_context_len is None else max_context_len
+            if window:
+                reach = min(reach, window + 63)
+            parts = max(1, min(-(-2 * self.num_cus // max(sets, 1)), -(-reach // 64))) if sets < self.num_cus else 1
+        ws_ml = ws_o = None
+        if parts > 1:
+            ws_ml = self.workspace("together_ml", tokens * H * parts * 2)
+            ws_o = self.workspace("together_o", tokens * parts * H * DV)
         self._done("attention_together", self.lib.atom_attention_together(
             _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), self._code(q), _ptr(token_seq), _ptr(positions),
             _ptr(block_tables), block_tables.shape[1], tokens, H, G, D, DV, page_size, ctypes.c_float(scale),
-            _ptr(head_scale), _ptr(sink), _ptr(talk), int(window or 0), self._stream()))
+            _ptr(head_scale), _ptr(sink), _ptr(talk), int(window or 0), int(parts), _ptr(ws_ml), _ptr(ws_o),
+            self._stream()))
         return out
 
     def router_choose(self, logits, correction, top: int, renormalize: bool = False):

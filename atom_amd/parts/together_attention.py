@@ -128,7 +128,8 @@ class TogetherAttention(Mixer):
         out = torch.empty((T, H, DV), dtype=ctx.dtype, device=x.device)
         ops.attention_together(q, pages.k_cache, pages.v_cache, out, ctx.token_seq, ctx.positions,
                                ctx.block_tables[group], self.scale, head_scale=self.p("temp"), sink=self.p("sink"),
-                               talk=self.p("talk"), window=self.window, max_context_len=ctx.max_context_len)
+                               talk=self.p("talk"), window=self.window, max_context_len=ctx.max_context_len,
+                               cu_seqlens_q=ctx.cu_seqlens_q, max_q_len=ctx.max_q_len)
         return ops.linear(out.view(T, H * DV), self.params["o.weight"], self.p("o.bias"), out_dtype=torch.float32)
 
 

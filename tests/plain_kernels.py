@@ -195,7 +195,8 @@ class PlainKernels:
         return q_out
 
     def attention_together(self, q, k_cache, v_cache, out, token_seq, positions, block_tables, scale, head_scale=None,
-                           sink=None, talk=None, window=None, max_context_len=None):
+                           sink=None, talk=None, window=None, max_context_len=None, cu_seqlens_q=None, max_q_len=None,
+                           parts=None):
         tokens, H, D = q.shape
         G, page_size = k_cache.shape[1], k_cache.shape[2]
         for t in range(tokens):

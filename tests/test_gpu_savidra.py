@@ -163,36 +163,82 @@ def _paged(keys, values, page, dtype, order_seed):
     return k_cache.to(DEV), v_cache.to(DEV), perm
 
 
-def _attend(ops, q, keys, values, positions, page, dtype, scale, temp=None, sink=None, talk=None, seed=0):
+def _attend(ops, q, keys, values, positions, page, dtype, scale, temp=None, sink=None, talk=None, seed=0, how="blocks"):
+    """``how``: "blocks" (a block a token and set of heads), "parts" (a token's keys cut over three blocks), "tiles"
+    (the rows as a prompt portion of one request: the matrix cores where the sizes allow)."""
     T, H, D = q.shape
     k_cache, v_cache, perm = _paged(keys, values, page, dtype, seed)
     out = torch.empty((T, H, values.shape[2]), dtype=dtype, device=DEV)
     dev = lambda t: f32(t) if t is not None else None  # noqa: E731
+    more = {"blocks": dict(parts=1), "parts": dict(parts=3), "tiles": dict(cu_seqlens_q=i32([0, T]), max_q_len=T)}[how]
     ops.attention_together(q.to(dtype).to(DEV), k_cache, v_cache, out, i32([0] * T), i32(positions), i32([perm]), scale,
-                           head_scale=dev(temp), sink=dev(sink), talk=dev(talk), max_context_len=keys.shape[0])
+                           head_scale=dev(temp), sink=dev(sink), talk=dev(talk), max_context_len=keys.shape[0], **more)
     return out
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("how", ["blocks", "parts", "tiles"])
 @pytest.mark.parametrize("H,G,D,DV,page,n,sink,talk,temp", [
     (4, 2, 10, 6, 4, 70, True, False, False), (6, 3, 6, 4, 16, 131, False, True, True), (2, 1, 12, 20, 8, 64, True, True, True),
     (4, 2, 128, 32, 16, 300, True, False, False), (4, 2, 48, 32, 16, 257, False, True, True), (1, 1, 14, 3, 16, 65, False, True, False),
-    (16, 4, 64, 64, 16, 200, False, True, True), (3, 3, 7, 7, 4, 5, False, False, False)])
-def test_attention_against_plain(dtype, H, G, D, DV, page, n, sink, talk, temp):
+    (16, 4, 64, 64, 16, 200, False, True, True), (3, 3, 7, 7, 4, 5, False, False, False), (8, 2, 128, 128, 16, 300, False, True, True),
+    (8, 8, 64, 128, 8, 100, True, True, False), (12, 3, 64, 32, 4, 90, True, False, True), (32, 2, 128, 64, 16, 150, True, False, False)])
+def test_attention_against_plain(dtype, how, H, G, D, DV, page, n, sink, talk, temp):
     ops = gpu_ops()
     q, keys, values = rnd((n, H, D), 1).to(dtype), rnd((n, G, D), 2).to(dtype), rnd((n, G, DV), 3).to(dtype)
     sk = 1.5 * rnd((H,), 4) if sink else None
     tk = torch.eye(H) + 0.3 * rnd((H, H), 5) if talk else None
     tp = 1 + 0.3 * rnd((H,), 6) if temp else None
     rows = sorted({0, 1, 2, page - 1, page, n // 2, 63, 64, 65, n - 2, n - 1} & set(range(n)))
+    if how == "tiles":       # more than a tile of rows, the last tile not full
+        rows = sorted(set(rows) | set(range(max(0, n - 40), n, 2)))
     at = torch.tensor(rows)
     w = ps.softmax_weights(q[rows].double(), keys.double(), at, torch.arange(n), 0.3,
                            sink=sk.double() if sink else None, temp=tp.double() if temp else None)
     if talk:
         w = torch.einsum("hg,gij->hij", tk.double(), w)
     want = ps.apply_weights(w, values.double(), H).view(len(rows), H, DV)
-    got = _attend(ops, q[rows], keys, values, rows, page, dtype, 0.3, tp, sk, tk, seed=n)
+    got = _attend(ops, q[rows], keys, values, rows, page, dtype, 0.3, tp, sk, tk, seed=n, how=how)
     close(got, want, dtype, "attention")
+
+
+@pytest.mark.parametrize("talk", [False, True])
+def test_tiles_of_several_requests(talk):
+    """Portions of three requests and a single token in one launch, each behind a different number of cached tokens:
+    every block finds its request and tile from its index alone."""
+    ops = gpu_ops()
+    H, G, D, DV, page, dtype = 4, 2, 64, 32, 16, torch.bfloat16
+    lens, cached = [37, 1, 16, 50], [5, 80, 0, 100]
+    tk = torch.eye(H) + 0.3 * rnd((H, H), 5) if talk else None
+    blocks = [-(-(c + n) // page) for n, c in zip(lens, cached)]
+    k_cache = torch.zeros((sum(blocks) + 1, G, page, D), dtype=dtype)
+    v_cache = torch.zeros((sum(blocks) + 1, G, DV, page), dtype=dtype)
+    tables = torch.zeros((4, max(blocks)), dtype=torch.int32)
+    qs, wants, positions, seq_of, at = [], [], [], [], 1
+    for r, (n, c) in enumerate(zip(lens, cached)):
+        keys, values = rnd((c + n, G, D), 10 + r).to(dtype), rnd((c + n, G, DV), 20 + r).to(dtype)
+        tables[r, :blocks[r]] = torch.arange(at, at + blocks[r])
+        for j in range(c + n):
+            k_cache[at + j // page, :, j % page] = keys[j]
+            v_cache[at + j // page, :, :, j % page] = values[j]
+        at += blocks[r]
+        q = rnd((n, H, D), 30 + r).to(dtype)
+        pos = torch.arange(c, c + n)
+        w = ps.softmax_weights(q.double(), keys.double(), pos, torch.arange(c + n), 0.2)
+        if talk:
+            w = torch.einsum("hg,gij->hij", tk.double(), w)
+        wants.append(ps.apply_weights(w, values.double(), H).view(n, H, DV))
+        qs.append(q)
+        positions += pos.tolist()
+        seq_of += [r] * n
+    cu = [0]
+    for n in lens:
+        cu.append(cu[-1] + n)
+    out = torch.empty((sum(lens), H, DV), dtype=dtype, device=DEV)
+    ops.attention_together(torch.cat(qs).to(DEV), k_cache.to(DEV), v_cache.to(DEV), out, i32(seq_of), i32(positions),
+                           tables.to(DEV), 0.2, talk=f32(tk) if talk else None, max_context_len=150, cu_seqlens_q=i32(cu),
+                           max_q_len=max(lens))
+    close(out, torch.cat(wants), dtype, "tiles of several requests")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -206,8 +252,9 @@ def test_a_far_key_is_found_and_a_later_one_is_not(dtype, far):
     q = 0.1 * rnd((1, H, D), 3)
     q[0, :, 0], keys[far, 0, 0] = 6.0, 6.0
     values[far, 0] = 50.0
-    got = _attend(ops, q, keys, values, [n - 1], page, dtype, 1.0)
-    assert float(got.float().min()) > 45.0
+    for how in ("blocks", "parts"):
+        got = _attend(ops, q, keys, values, [n - 1], page, dtype, 1.0, how=how)
+        assert float(got.float().min()) > 45.0, how
     got = _attend(ops, q, keys, values, [far - 1], page, dtype, 1.0) if far else None
     assert got is None or float(got.float().abs().max()) < 10.0
     # a sink as large as the key's score takes half of the weight and brings no value
