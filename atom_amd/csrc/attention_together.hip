@@ -93,6 +93,36 @@ __device__ __forceinline__ void together_scores(const TogetherArgs& a, const T* 
   }
 }
 
+// sum over the keys lo .. hi of wr[key] * v(key) for one (value head, entry) whose row starts row_off elements into a
+// page: the value pages hold a page's keys contiguously, 16 bytes of them a load where the run allows it.  pages[]
+// holds the page of every page-sized run of the chunk, counted from the run that holds `base` (so that no look-up
+// in the block table stands between a thread and its loads).
+template <typename T>
+__device__ __forceinline__ float together_values(const T* __restrict__ v_cache, size_t page_stride, size_t row_off,
+                                                 const int* pages, const float* wr, int base, int lo, int hi,
+                                                 int page_size, float sum) {
+  const int run0 = base / page_size;
+  for (int key = lo; key <= hi;) {
+    const int page = pages[key / page_size - run0], off = key % page_size;
+    int run = page_size - off;
+    if (run > hi - key + 1) run = hi - key + 1;
+    const T* vr = v_cache + (size_t)page * page_stride + row_off + off;
+    int u = 0;
+    if (sizeof(T) == 2 && page_size % 8 == 0) {
+      union Pack { uint4 raw; bf16_t e[8]; };
+      for (; u + 8 <= run && (off + u) % 8 == 0; u += 8) {
+        Pack p;
+        p.raw = *reinterpret_cast<const uint4*>(vr + u);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sum += wr[key + u + e] * to_f32(p.e[e]);
+      }
+    }
+    for (; u < run; ++u) sum += wr[key + u] * to_f32(vr[u]);
+    key += run;
+  }
+  return sum;
+}
+
 template <typename T>
 __global__ void __launch_bounds__(kTogetherThreads)
 attention_together_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
@@ -106,6 +136,7 @@ attention_together_kernel(const T* __restrict__ q, const T* __restrict__ k_cache
   float* mixed = s + (size_t)HB * kTogetherChunk;   // HB * chunk: mixed weights (talk only)
   float* top = mixed + (a.talk != nullptr ? (size_t)HB * kTogetherChunk : 0);   // HB: running maximum
   float* den = top + HB;                            // HB: running sum, later its inverse
+  int* pg = reinterpret_cast<int*>(den + HB);       // chunk: the pages of the chunk's runs of keys
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1), wave = tid / kWave;
   constexpr int waves = kTogetherThreads / kWave;
@@ -163,6 +194,7 @@ attention_together_kernel(const T* __restrict__ q, const T* __restrict__ k_cache
     const int lo = base > first ? base : first;
     const int hi = base + kTogetherChunk - 1 < pos ? base + kTogetherChunk - 1 : pos;
     together_scores(a, k_cache, table, qs, s, h0, HB, base, lo, hi);
+    for (int r = tid; r <= hi / a.page_size - base / a.page_size; r += kTogetherThreads) pg[r] = table[base / a.page_size + r];
     // a thread turns the scores it wrote itself into weights
     for (int item = tid; item < HB * kTogetherChunk; item += kTogetherThreads) {
       const int hh = item / kTogetherChunk;
@@ -188,16 +220,8 @@ attention_together_kernel(const T* __restrict__ q, const T* __restrict__ k_cache
         const int hh = e / a.DV, i = e - hh * a.DV;
         const int kvh = (h0 + hh) / group;
         const float* wr = w + hh * kTogetherChunk - base;   // wr[key]
-        float sum = acc[r];
-        for (int key = lo; key <= hi;) {
-          const int page = table[key / a.page_size], off = key % a.page_size;
-          int run = a.page_size - off;
-          if (run > hi - key + 1) run = hi - key + 1;
-          const T* vr = v_cache + (((size_t)page * a.G + kvh) * a.DV + i) * (size_t)a.page_size + off;
-          for (int u = 0; u < run; ++u) sum += wr[key + u] * to_f32(vr[u]);
-          key += run;
-        }
-        acc[r] = sum;
+        acc[r] = together_values(v_cache, (size_t)a.G * a.DV * a.page_size, ((size_t)kvh * a.DV + i) * a.page_size, pg, wr,
+                                 base, lo, hi, a.page_size, acc[r]);
       }
     }
     __syncthreads();   // s and mixed are rewritten by the next chunk
@@ -224,6 +248,7 @@ attention_together_part_kernel(const T* __restrict__ q, const T* __restrict__ k_
   float* mixed = s + (size_t)HB * kTogetherChunk;
   float* top = mixed + (a.talk != nullptr ? (size_t)HB * kTogetherChunk : 0);
   float* den = top + HB;
+  int* pg = reinterpret_cast<int*>(den + HB);
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1), wave = tid / kWave;
   constexpr int waves = kTogetherThreads / kWave;
@@ -293,6 +318,7 @@ attention_together_part_kernel(const T* __restrict__ q, const T* __restrict__ k_
     const int lo = base > first ? base : first;
     const int hi = base + kTogetherChunk - 1 < pos ? base + kTogetherChunk - 1 : pos;
     together_scores(a, k_cache, table, qs, s, h0, HB, base, lo, hi);
+    for (int r = tid; r <= hi / a.page_size - base / a.page_size; r += kTogetherThreads) pg[r] = table[base / a.page_size + r];
     for (int item = tid; item < HB * kTogetherChunk; item += kTogetherThreads) {
       const int hh = item / kTogetherChunk;
       s[item] = expf(s[item] - top[hh]) * den[hh];
@@ -317,16 +343,8 @@ attention_together_part_kernel(const T* __restrict__ q, const T* __restrict__ k_
         const int hh = e / a.DV, i = e - hh * a.DV;
         const int kvh = (h0 + hh) / group;
         const float* wr = w + hh * kTogetherChunk - base;
-        float sum = acc[r];
-        for (int key = lo; key <= hi;) {
-          const int page = table[key / a.page_size], off = key % a.page_size;
-          int run = a.page_size - off;
-          if (run > hi - key + 1) run = hi - key + 1;
-          const T* vr = v_cache + (((size_t)page * a.G + kvh) * a.DV + i) * (size_t)a.page_size + off;
-          for (int u = 0; u < run; ++u) sum += wr[key + u] * to_f32(vr[u]);
-          key += run;
-        }
-        acc[r] = sum;
+        acc[r] = together_values(v_cache, (size_t)a.G * a.DV * a.page_size, ((size_t)kvh * a.DV + i) * a.page_size, pg, wr,
+                                 base, lo, hi, a.page_size, acc[r]);
       }
     }
     __syncthreads();
@@ -351,7 +369,7 @@ __global__ void together_sum_parts_kernel(const float* __restrict__ ws_o, T* __r
 
 static size_t together_lds(int H, int G, int D, bool talk) {
   const int HB = talk ? H : H / G;
-  return ((size_t)HB * D + (size_t)HB * kTogetherChunk * (talk ? 2 : 1) + 2 * (size_t)HB) * sizeof(float);
+  return ((size_t)HB * D + (size_t)HB * kTogetherChunk * (talk ? 2 : 1) + 2 * (size_t)HB + kTogetherChunk) * sizeof(float);
 }
 
 ATOM_EXPORT int atom_attention_together(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,

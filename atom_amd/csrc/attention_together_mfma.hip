@@ -13,7 +13,8 @@
 // is the B operand of the second.  The keys are walked twice: once for every (query, head)'s maximum and sum, which
 // are per-lane numbers, then for the finished weights.  Mixing the heads is entrywise in this layout: the waves
 // exchange their heads' weights of a chunk through LDS (two buffers in turn, one barrier a chunk) and every wave
-// forms sum_g talk[h, g] w_g for its own heads.  Chunks are counted from position 0.
+// forms sum_g talk[h, g] w_g for its own heads.  Chunks are counted from position 0.  A chunk's key rows are asked for
+// one chunk ahead of their use and its value rows before its scores are formed, so a wave waits for memory less.
 //
 // A block finds its request and tile from the block index alone: tile j of request s has the place
 // cu[s] / 16 + s + j, which is unique, so the launch needs no list of tiles from the host.
@@ -91,32 +92,64 @@ together_tile_kernel(TogetherTileArgs a) {
     hs[u] = a.scale_log2 * (a.head_scale != nullptr ? a.head_scale[h] : 1.f);
   }
 
-  // scores of head u against the 16 keys from base, in the exp2 domain, -inf where the lane's query does not see the key
-  auto scores = [&](int u, int base) -> tg_f32x4 {
+  // The 16 key rows from base as this lane's part of the A operand of the first product (head u's key/value head).
+  struct KeyRows { tg_bf16x8 f[D / 32]; };
+  auto load_keys = [&](int u, int base) -> KeyRows {
     const int h = h0 + wave + kTileWaves * u;
-    int key = base + n;                       // the key row this lane brings to the A operand
-    if (key > pos_hi) key = pos_hi;           // beyond the tile's last key: any valid row, masked below
+    int key = base + n;                       // the key row this lane brings
+    if (key > pos_hi) key = pos_hi;           // beyond the tile's last key: any valid row, masked in the scores
     const int page = table[key / ps], off = key - key / ps * ps;
     const bf16_t* kr = a.k_cache + (((size_t)page * a.G + h / group) * ps + off) * (size_t)D + 8 * g4;
+    KeyRows k;
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j) k.f[j] = *reinterpret_cast<const tg_bf16x8*>(kr + 32 * j);
+    return k;
+  };
+  // scores of head u against those keys, in the exp2 domain, -inf where the lane's query does not see the key
+  auto scores = [&](int u, const KeyRows& k, int base) -> tg_f32x4 {
     tg_f32x4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < D / 32; ++j)
-      s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const tg_bf16x8*>(kr + 32 * j), qf[u][j], s, 0, 0, 0);
+    for (int j = 0; j < D / 32; ++j) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k.f[j], qf[u][j], s, 0, 0, 0);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int k = base + 4 * g4 + i;
-      s[i] = (k >= first_row && k <= pos) ? s[i] * hs[u] : -INFINITY;
+      const int key = base + 4 * g4 + i;
+      s[i] = (key >= first_row && key <= pos) ? s[i] * hs[u] : -INFINITY;
     }
     return s;
   };
+  // The values of the four keys from base + 4 g4, rows n + 16 t of head u's value head: the A operand of the second
+  // product.  One page holds the four.
+  struct ValueRows { tg_bf16x4 f[NDV]; };
+  auto load_values = [&](int u, int base) -> ValueRows {
+    int key0 = base + 4 * g4;
+    if (key0 > pos_hi) key0 = pos_hi & ~3;      // unseen by every query: any valid place, the weights are zero
+    const int page = table[key0 / ps], off = key0 - key0 / ps * ps;
+    const int kvh = (h0 + wave + kTileWaves * u) / group;
+    const bf16_t* vr = a.v_cache + (((size_t)page * a.G + kvh) * DV + n) * (size_t)ps + off;
+    ValueRows v;
+#pragma unroll
+    for (int t = 0; t < NDV; ++t) v.f[t] = *reinterpret_cast<const tg_bf16x4*>(vr + (size_t)16 * t * ps);
+    return v;
+  };
 
   const int start = first_blk / kTileRows * kTileRows;
-  // every (query, head)'s maximum and sum
+  // every (query, head)'s maximum and sum; the next chunk's key rows are asked for before this chunk's are used
+  KeyRows ahead[HPW];
+#pragma unroll
+  for (int u = 0; u < HPW; ++u)
+    if (own[u]) ahead[u] = load_keys(u, start);
   for (int base = start; base <= pos_hi; base += kTileRows) {
+    KeyRows now[HPW];
 #pragma unroll
     for (int u = 0; u < HPW; ++u) {
       if (!own[u]) continue;
-      const tg_f32x4 s = scores(u, base);
+      now[u] = ahead[u];
+      if (base + kTileRows <= pos_hi) ahead[u] = load_keys(u, base + kTileRows);
+    }
+#pragma unroll
+    for (int u = 0; u < HPW; ++u) {
+      if (!own[u]) continue;
+      const tg_f32x4 s = scores(u, now[u], base);
       const float cm = rows_max(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
       const float m_new = fmaxf(top[u], cm);
       // no branch around the exchange between lanes: a query that has seen no key yet keeps a sum of zero
@@ -146,14 +179,26 @@ together_tile_kernel(TogetherTileArgs a) {
   for (int u = 0; u < HPW; ++u)
 #pragma unroll
     for (int t = 0; t < NDV; ++t) acc[u][t] = tg_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int u = 0; u < HPW; ++u)
+    if (own[u]) ahead[u] = load_keys(u, start);
   int turn = 0;
   for (int base = start; base <= pos_hi; base += kTileRows, turn ^= 1) {
+    KeyRows now[HPW];
+    ValueRows vals[HPW];
+#pragma unroll
+    for (int u = 0; u < HPW; ++u) {
+      if (!own[u]) continue;
+      now[u] = ahead[u];
+      vals[u] = load_values(u, base);          // in flight while the scores are formed
+      if (base + kTileRows <= pos_hi) ahead[u] = load_keys(u, base + kTileRows);
+    }
     tg_f32x4 w[HPW];
 #pragma unroll
     for (int u = 0; u < HPW; ++u) {
       w[u] = tg_f32x4{0.f, 0.f, 0.f, 0.f};
       if (!own[u]) continue;
-      const tg_f32x4 s = scores(u, base);
+      const tg_f32x4 s = scores(u, now[u], base);
 #pragma unroll
       for (int i = 0; i < 4; ++i) w[u][i] = exp2f(s[i] - top[u]) * den[u];   // exp2(-inf) = 0 where unseen
       if (mixes) pbuf[turn][wave + kTileWaves * u][lane] = w[u];
@@ -173,24 +218,16 @@ together_tile_kernel(TogetherTileArgs a) {
         w[u] = m;
       }
     }
-    // the four keys this lane brings to the A operand of the second product: one page holds them
-    int key0 = base + 4 * g4;
-    if (key0 > pos_hi) key0 = pos_hi & ~3;      // unseen by every query: any valid place, the weights are zero
-    const int page = table[key0 / ps], off = key0 - key0 / ps * ps;
 #pragma unroll
     for (int u = 0; u < HPW; ++u) {
       if (!own[u]) continue;
-      const int kvh = (h0 + wave + kTileWaves * u) / group;
       tg_bf16x4 pb;
 #pragma unroll
       for (int i = 0; i < 4; ++i) pb[i] = (__bf16)w[u][i];
-      const bf16_t* vr = a.v_cache + (((size_t)page * a.G + kvh) * DV + n) * (size_t)ps + off;
 #pragma unroll
-      for (int t = 0; t < NDV; ++t) {
-        const tg_bf16x4 vf = *reinterpret_cast<const tg_bf16x4*>(vr + (size_t)16 * t * ps);
-        acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(tg_s16x4, vf),
+      for (int t = 0; t < NDV; ++t)
+        acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(tg_s16x4, vals[u].f[t]),
                                                               __builtin_bit_cast(tg_s16x4, pb), acc[u][t], 0, 0, 0);
-      }
     }
   }
   if (!row_ok) return;

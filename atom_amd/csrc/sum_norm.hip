@@ -20,8 +20,8 @@ struct SumTerms {
   int n;
 };
 
-__device__ __forceinline__ float term_at(const SumTerms& s, int i, size_t at) {
-  return s.dtype[i] == ATOM_F32 ? static_cast<const float*>(s.y[i])[at] : to_f32(static_cast<const bf16_t*>(s.y[i])[at]);
+__device__ __forceinline__ float term_at(const void* y, int dtype, size_t at) {
+  return dtype == ATOM_F32 ? static_cast<const float*>(y)[at] : to_f32(static_cast<const bf16_t*>(y)[at]);
 }
 
 template <typename T>
@@ -34,7 +34,10 @@ sum_norm_kernel(float* __restrict__ stream, float alpha, SumTerms terms, const f
   float ss = 0.f;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     float v = alpha != 0.f ? alpha * stream[base + i] : 0.f;
-    for (int k = 0; k < terms.n; ++k) v += terms.scale[k] * term_at(terms, k, base + i);
+    // the terms by constant index, so that the argument's arrays stay in scalar registers
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if (k < terms.n) v += terms.scale[k] * term_at(terms.y[k], terms.dtype[k], base + i);
     row[i] = v;
     ss += v * v;
   }
