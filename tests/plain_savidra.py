@@ -117,7 +117,7 @@ class PlainSavidra:
 
     # ---- mixers
 
-    def _left(self, i, m, h, positions, mem, p, biased=True, conv=True, talk=True):
+    def _project(self, m, h, positions, mem, p, biased=True, conv=True):
         w, eps = self.w, self.eps
         H, G, D, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
         T = h.shape[0]
@@ -178,7 +178,7 @@ class PlainSavidra:
         w, mem, m = self.w, self.mem[i], layer["mixer"]
         p = f"l{i}.mix"
         if layer["type"] == "attention":
-            q, k, v = self._left(i, m, h, positions, mem, p, biased=False, conv=False)
+            q, k, v = self._project(m, h, positions, mem, p, biased=False, conv=False)
             if m.get("v_mix"):
                 if "v_first" in shared:
                     lam = w[f"{p}.vmix"]
@@ -190,7 +190,7 @@ class PlainSavidra:
         if layer["type"] != "parallel":
             raise ValueError(layer["type"])
         lm = m["left"]
-        q, k, v = self._left(i, lm, h, positions, mem, f"{p}.left")
+        q, k, v = self._project(lm, h, positions, mem, f"{p}.left")
         o = self._attend(mem, q, k, v, positions, lm["scale"], lm["heads"], temp=w[f"{p}.left.temp"],
                          talk=w[f"{p}.left.talk"])
         left = o @ w[f"{p}.left.o"].T + w[f"{p}.left.o.b"]
