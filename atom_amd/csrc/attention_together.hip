@@ -367,6 +367,18 @@ __global__ void together_sum_parts_kernel(const float* __restrict__ ws_o, T* __r
   out[idx] = from_f32<T>(sum);
 }
 
+ATOM_EXPORT int atom_together_sum_parts(const float* ws_o, void* out, int dtype, int parts, int tokens, int row,
+                                        hipStream_t stream) {
+  if (ws_o == nullptr || out == nullptr || parts < 1 || tokens < 0 || row <= 0) return ATOM_BAD_SHAPE;
+  const size_t total = (size_t)tokens * row;
+  if (total == 0) return ATOM_OK;
+  const size_t blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffffu) return ATOM_TOO_LARGE;
+  ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((together_sum_parts_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream,
+                                                 ws_o, (T*)out, parts, row, total));
+  return launch_status();
+}
+
 static size_t together_lds(int H, int G, int D, bool talk) {
   const int HB = talk ? H : H / G;
   return ((size_t)HB * D + (size_t)HB * kTogetherChunk * (talk ? 2 : 1) + 2 * (size_t)HB + kTogetherChunk) * sizeof(float);

@@ -16,6 +16,9 @@
 // forms sum_g talk[h, g] w_g for its own heads.  Chunks are counted from position 0.  A chunk's key rows are asked for
 // one chunk ahead of their use and its value rows before its scores are formed, so a wave waits for memory less.
 //
+// Where the tiles alone would leave the chip idle, a tile's chunks are cut over `parts` blocks (three launches, as in
+// attention_together.hip: maxima and sums, shares of the weighted sum, their sum in the order of the parts).
+//
 // A block finds its request and tile from the block index alone: tile j of request s has the place
 // cu[s] / 16 + s + j, which is unique, so the launch needs no list of tiles from the host.
 #include "common.h"
@@ -34,9 +37,14 @@ struct TogetherTileArgs {
   int max_blocks, num_seqs, H, G, page_size, window;
   float scale_log2;
   const float* head_scale; const float* sink; const float* talk;
+  int parts;          // > 1: a tile's chunks are cut over this many blocks (grid z), in three launches
+  float* ws_ml;       // [tokens, H, parts, 2]: a part's maximum (exp2 domain) and sum
+  float* ws_o;        // [tokens, parts, H, DV]: a part's share of the weighted sum
 };
 
-template <int D, int NDV, int HPW>
+// PASS 0: both walks over all of the tile's chunks.  PASS 1: the maximum and sum of this part's chunks.  PASS 2: the
+// parts' maxima and sums merged in the order of the parts, then this part's share of the weighted sum.
+template <int D, int NDV, int HPW, int PASS>
 __global__ void __launch_bounds__(kTileWaves * kWave)
 together_tile_kernel(TogetherTileArgs a) {
   constexpr int DV = 16 * NDV;
@@ -132,19 +140,28 @@ together_tile_kernel(TogetherTileArgs a) {
     return v;
   };
 
-  const int start = first_blk / kTileRows * kTileRows;
-  // every (query, head)'s maximum and sum; the next chunk's key rows are asked for before this chunk's are used
+  int start = first_blk / kTileRows * kTileRows;
+  int stop = pos_hi + 1;                       // chunks from start up to, not including, stop
+  if (PASS != 0) {
+    const int chunks = (pos_hi - start) / kTileRows + 1;
+    const int each = (chunks + a.parts - 1) / a.parts;
+    const int c0 = blockIdx.z * each, c1 = c0 + each < chunks ? c0 + each : chunks;
+    stop = start + c1 * kTileRows;
+    start += c0 * kTileRows;                   // start >= stop: this part has no chunk
+  }
   KeyRows ahead[HPW];
+  if (PASS != 2) {
+  // every (query, head)'s maximum and sum; the next chunk's key rows are asked for before this chunk's are used
 #pragma unroll
   for (int u = 0; u < HPW; ++u)
-    if (own[u]) ahead[u] = load_keys(u, start);
-  for (int base = start; base <= pos_hi; base += kTileRows) {
+    if (own[u] && start < stop) ahead[u] = load_keys(u, start);
+  for (int base = start; base < stop; base += kTileRows) {
     KeyRows now[HPW];
 #pragma unroll
     for (int u = 0; u < HPW; ++u) {
       if (!own[u]) continue;
       now[u] = ahead[u];
-      if (base + kTileRows <= pos_hi) ahead[u] = load_keys(u, base + kTileRows);
+      if (base + kTileRows < stop) ahead[u] = load_keys(u, base + kTileRows);
     }
 #pragma unroll
     for (int u = 0; u < HPW; ++u) {
@@ -157,6 +174,30 @@ together_tile_kernel(TogetherTileArgs a) {
       const float part = exp2f(s[0] - m_at) + exp2f(s[1] - m_at) + exp2f(s[2] - m_at) + exp2f(s[3] - m_at);
       den[u] = den[u] * exp2f(top[u] - m_at) + rows_sum(part);
       top[u] = m_new;
+    }
+  }
+  }
+  if (PASS == 1) {
+    if (row_ok && g4 == 0) {
+#pragma unroll
+      for (int u = 0; u < HPW; ++u) {
+        if (!own[u]) continue;
+        float* ml = a.ws_ml + (((size_t)(t0 + n) * a.H + h0 + wave + kTileWaves * u) * a.parts + blockIdx.z) * 2;
+        ml[0] = top[u], ml[1] = den[u];
+      }
+    }
+    return;
+  }
+  if (PASS == 2 && row_ok) {
+#pragma unroll
+    for (int u = 0; u < HPW; ++u) {
+      if (!own[u]) continue;
+      const float* ml = a.ws_ml + ((size_t)(t0 + n) * a.H + h0 + wave + kTileWaves * u) * a.parts * 2;
+      float m = -INFINITY, l = 0.f;
+      for (int p = 0; p < a.parts; ++p) m = fmaxf(m, ml[2 * p]);
+      for (int p = 0; p < a.parts; ++p)
+        if (ml[2 * p] != -INFINITY) l += ml[2 * p + 1] * exp2f(ml[2 * p] - m);
+      top[u] = m, den[u] = l;
     }
   }
 #pragma unroll
@@ -181,9 +222,9 @@ together_tile_kernel(TogetherTileArgs a) {
     for (int t = 0; t < NDV; ++t) acc[u][t] = tg_f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int u = 0; u < HPW; ++u)
-    if (own[u]) ahead[u] = load_keys(u, start);
+    if (own[u] && start < stop) ahead[u] = load_keys(u, start);
   int turn = 0;
-  for (int base = start; base <= pos_hi; base += kTileRows, turn ^= 1) {
+  for (int base = start; base < stop; base += kTileRows, turn ^= 1) {
     KeyRows now[HPW];
     ValueRows vals[HPW];
 #pragma unroll
@@ -191,7 +232,7 @@ together_tile_kernel(TogetherTileArgs a) {
       if (!own[u]) continue;
       now[u] = ahead[u];
       vals[u] = load_values(u, base);          // in flight while the scores are formed
-      if (base + kTileRows <= pos_hi) ahead[u] = load_keys(u, base + kTileRows);
+      if (base + kTileRows < stop) ahead[u] = load_keys(u, base + kTileRows);
     }
     tg_f32x4 w[HPW];
 #pragma unroll
@@ -234,7 +275,14 @@ together_tile_kernel(TogetherTileArgs a) {
 #pragma unroll
   for (int u = 0; u < HPW; ++u) {
     if (!own[u]) continue;
-    bf16_t* dst = a.out + ((size_t)(t0 + n) * a.H + h0 + wave + kTileWaves * u) * DV + 4 * g4;
+    const int h = h0 + wave + kTileWaves * u;
+    if (PASS == 2) {
+      float* dst = a.ws_o + (((size_t)(t0 + n) * a.parts + blockIdx.z) * a.H + h) * DV + 4 * g4;
+#pragma unroll
+      for (int t = 0; t < NDV; ++t) *reinterpret_cast<tg_f32x4*>(dst + 16 * t) = acc[u][t];
+      continue;
+    }
+    bf16_t* dst = a.out + ((size_t)(t0 + n) * a.H + h) * DV + 4 * g4;
 #pragma unroll
     for (int t = 0; t < NDV; ++t) {
       tg_bf16x4 o;
@@ -254,12 +302,22 @@ ATOM_EXPORT int atom_attention_together_tiles_supports(int H, int G, int D, int 
   return (H > 0 && G > 0 && H % G == 0 && together_tile_takes(H, G, D, DV, page_size, mixes != 0)) ? 1 : 0;
 }
 
+template <int D, int NDV, int HPW>
+static void together_tile_passes(const TogetherTileArgs& a, dim3 grid, hipStream_t stream) {
+  const dim3 block(kTileWaves * kWave);
+  if (a.parts == 1) {
+    hipLaunchKernelGGL((together_tile_kernel<D, NDV, HPW, 0>), grid, block, 0, stream, a);
+  } else {
+    hipLaunchKernelGGL((together_tile_kernel<D, NDV, HPW, 1>), grid, block, 0, stream, a);
+    hipLaunchKernelGGL((together_tile_kernel<D, NDV, HPW, 2>), grid, block, 0, stream, a);
+  }
+}
+
 template <int D, int NDV>
 static int together_tile_launch(const TogetherTileArgs& a, dim3 grid, int HB, hipStream_t stream) {
-  const dim3 block(kTileWaves * kWave);
-  if (HB <= 4) hipLaunchKernelGGL((together_tile_kernel<D, NDV, 1>), grid, block, 0, stream, a);
-  else if (HB <= 8) hipLaunchKernelGGL((together_tile_kernel<D, NDV, 2>), grid, block, 0, stream, a);
-  else hipLaunchKernelGGL((together_tile_kernel<D, NDV, 4>), grid, block, 0, stream, a);
+  if (HB <= 4) together_tile_passes<D, NDV, 1>(a, grid, stream);
+  else if (HB <= 8) together_tile_passes<D, NDV, 2>(a, grid, stream);
+  else together_tile_passes<D, NDV, 4>(a, grid, stream);
   return launch_status();
 }
 
@@ -267,18 +325,20 @@ ATOM_EXPORT int atom_attention_together_tiles(const void* q, const void* k_cache
                                               const int* cu_q, const int* positions, const int* block_tables,
                                               int max_blocks, int tokens, int num_seqs, int H, int G, int D, int DV,
                                               int page_size, float scale, const float* head_scale, const float* sink,
-                                              const float* talk, int window, hipStream_t stream) {
+                                              const float* talk, int window, int parts, float* ws_ml, float* ws_o,
+                                              hipStream_t stream) {
   if (tokens < 0 || num_seqs <= 0 || H <= 0 || G <= 0 || H % G || max_blocks <= 0 || window < 0) return ATOM_BAD_SHAPE;
   if (q == nullptr || k_cache == nullptr || v_cache == nullptr || out == nullptr) return ATOM_BAD_SHAPE;
   if (cu_q == nullptr || positions == nullptr || block_tables == nullptr) return ATOM_BAD_SHAPE;
   const bool mixes = talk != nullptr;
   if (!together_tile_takes(H, G, D, DV, page_size, mixes)) return ATOM_UNSUPPORTED;
+  if (parts < 1 || parts > 65535 || (parts > 1 && (ws_ml == nullptr || ws_o == nullptr))) return ATOM_BAD_SHAPE;
   if (tokens == 0) return ATOM_OK;
   const int HB = mixes ? H : H / G;
   TogetherTileArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, cu_q, positions,
                      block_tables, max_blocks, num_seqs, H, G, page_size, window, scale * 1.4426950408889634f,
-                     head_scale, sink, talk};
-  const dim3 grid(tokens / kTileRows + num_seqs + 1, mixes ? 1 : G);
+                     head_scale, sink, talk, parts, ws_ml, ws_o};
+  const dim3 grid(tokens / kTileRows + num_seqs + 1, mixes ? 1 : G, parts);
 #define ATOM_TILE(DD, NN) return together_tile_launch<DD, NN>(a, grid, HB, stream)
   if (D == 64) {
     if (DV == 32) ATOM_TILE(64, 2);

@@ -199,7 +199,8 @@ class HipKernels:
                    "atom_step_decay", "atom_group_norm_gate", "atom_qkv_plain_write", "atom_narrow_heads",
                    "atom_mean_of_norms", "atom_embedding_positions", "atom_unary_act", "atom_stream_add", "atom_scale_rows",
                    "atom_stream_norm", "atom_sum_norm", "atom_shift_rows", "atom_qkv_rot_write",
-                   "atom_attention_together", "atom_attention_together_tiles", "atom_attention_together_tiles_supports"):
+                   "atom_attention_together", "atom_attention_together_tiles", "atom_attention_together_tiles_supports",
+                   "atom_together_sum_parts"):
             getattr(self.lib, fn).restype = ctypes.c_int
         self.allow_library_gemm = True
         # bfloat16 products of few rows run this library's own weight-streaming kernels: up to 64 rows, and
@@ -1727,10 +1728,22 @@ class HipKernels:
             self._check("cu_seqlens_q", cu_seqlens_q, torch.int32, (seqs + 1,))
             if block_tables.shape[0] != seqs:
                 raise KernelError("attention: one block table row per request is needed")
+            if parts is None:
+                # enough blocks for four a CU, every part with at least four chunks of 16 keys
+                blocks = (tokens // 16 + seqs + 1) * (1 if talk is not None else G)
+                reach = block_tables.shape[1] * page_size if max_context_len is None else max_context_len
+                parts = max(1, min(8, 4 * self.num_cus // blocks, reach // 64))
+            ws_ml = ws_o = None
+            if parts > 1:
+                ws_ml = self.workspace("together_ml", tokens * H * parts * 2)
+                ws_o = self.workspace("together_o", tokens * parts * H * DV)
             self._done("attention_together_tiles", self.lib.atom_attention_together_tiles(
                 _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(cu_seqlens_q), _ptr(positions), _ptr(block_tables),
                 block_tables.shape[1], tokens, seqs, H, G, D, DV, page_size, ctypes.c_float(scale), _ptr(head_scale),
-                _ptr(sink), _ptr(talk), int(window or 0), self._stream()))
+                _ptr(sink), _ptr(talk), int(window or 0), int(parts), _ptr(ws_ml), _ptr(ws_o), self._stream()))
+            if parts > 1:
+                self._done("together_sum_parts", self.lib.atom_together_sum_parts(
+                    _ptr(ws_o), _ptr(out), self._code(out), int(parts), tokens, H * DV, self._stream()))
             return out
         sets = tokens * (1 if talk is not None else G)
         if parts is None:

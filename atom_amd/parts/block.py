@@ -158,13 +158,15 @@ class NormedSumBlock(Block):
     ``x <- norm2(alpha x + ffn(x))`` (``feed_forward`` None leaves the second step out).  The sublayers read the
     stream, which is float32 and kept whole (nothing pending); its rows in the step's type, for the products that
     read them, come out of the kernel that norms it.  A mixer with ``reads_stream`` is handed the float32 rows.
-    ``names["mixer"]`` may be empty: the mixer then takes the layer's own prefix."""
+    ``names["mixer"]`` may be empty: the mixer then takes the layer's own prefix.  A checkpoint that holds the second
+    norm's weight for a layer without feed-forward gets the second step with nothing added: ``x <- norm2(alpha x)``."""
 
     def __init__(self, mixer: PartChoice, feed_forward: PartChoice | None, norm: PartChoice, alpha: float = 1.0,
                  prefix: str = "", names: dict[str, str] | None = None):
         super().__init__(prefix)
         n = {"mixer": "mix", "mixer_norm": "norm1", "ffn": "mlp", "ffn_norm": "norm2", **(names or {})}
         sub = lambda name: (f"{prefix}.{n[name]}" if prefix else n[name]) if n[name] else prefix  # noqa: E731
+        self._norm_choice, self._ffn_norm_prefix, self._ffn_norm_name = norm, sub("ffn_norm"), n["ffn_norm"]
         self.alpha = float(alpha)
         self._mixer = mixer.build(MIXERS, prefix=sub("mixer"))
         self.mixer_norm = norm.build(NORMS, prefix=sub("mixer_norm"))
@@ -179,7 +181,13 @@ class NormedSumBlock(Block):
         return self._mixer
 
     def children(self):
-        return [self._mixer, self.mixer_norm] + ([self.ffn, self.ffn_norm] if self.ffn is not None else [])
+        return ([self._mixer, self.mixer_norm] + ([self.ffn] if self.ffn is not None else [])
+                + ([self.ffn_norm] if self.ffn_norm is not None else []))
+
+    def adopt_shapes(self, shape_of):
+        named = shape_of(self._ffn_norm_name) is not None or shape_of(f"{self._ffn_norm_name}.weight") is not None
+        if self.ffn is None and self.ffn_norm is None and named:
+            self.ffn_norm = self._norm_choice.build(NORMS, prefix=self._ffn_norm_prefix)
 
     @staticmethod
     def _summands(ops, y):
@@ -206,6 +214,8 @@ class NormedSumBlock(Block):
         if self.ffn is not None:
             terms, scales = self._summands(ops, self.ffn.forward(ctx, reads))
             reads = self.ffn_norm.forward_sum(ctx, terms, scales, stream, self.alpha, copy=not self._mixer.reads_stream)
+        elif self.ffn_norm is not None:
+            reads = self.ffn_norm.forward_sum(ctx, [], [], stream, self.alpha, copy=not self._mixer.reads_stream)
         if reads is not stream:
             ctx.memo[("stream copy", stream.data_ptr())] = reads
         return stream, None

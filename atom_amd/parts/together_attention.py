@@ -65,9 +65,10 @@ class TogetherAttention(Mixer):
     def cache_need(self):
         pages = KVCacheNeed(self.num_kv_heads, self.head_dim, self.window, None,
                             self.value_dim if self.value_dim != self.head_dim else None)
-        if not self.conv_taps or self.conv_taps == 1:
+        if not self.conv_taps:
             return pages
-        return JointNeed((pages, StateNeed(((self.conv_taps - 1) * self.channels,), torch.float32)))
+        # one tap carries nothing; its row of one number keeps the convolution's kernel one for all tap counts
+        return JointNeed((pages, StateNeed((max(1, (self.conv_taps - 1) * self.channels),), torch.float32)))
 
     def param_specs(self):
         n, h = self.names, self.hidden_size
@@ -107,8 +108,6 @@ class TogetherAttention(Mixer):
             qkv = torch.empty((T, self.channels), dtype=torch.float32, device=x.device)
             ops.conv_silu_state(proj, self.channels, self.params["conv.weight"], carried.state, ctx.cu_seqlens_q,
                                 ctx.slot_of_seq, qkv, max_q_len=ctx.max_q_len, activation="none")
-        elif self.conv_taps == 1:
-            raise NotImplementedError("a convolution of one tap is a weight per channel; no model has asked for it")
         else:
             qkv = proj
         source = keep = None

@@ -134,10 +134,11 @@ class PlainSavidra:
         q = plain_norm(parts["q"].view(T, H, D), w[f"{p}.q.norm"], eps)
         k = plain_norm(parts["k"].view(T, G, D), w[f"{p}.k.norm"], eps)
         v = parts["v"].view(T, G, dv)
-        rot = m["rot"]
-        factor = (rot.get("scaling") or {}).get("factor", 1.0)
-        q = rotate_half(q, positions, rot["dims"], rot["base"], factor)
-        k = rotate_half(k, positions, rot["dims"], rot["base"], factor)
+        rot = m.get("rot")
+        if rot is not None:
+            factor = (rot.get("scaling") or {}).get("factor", 1.0)
+            q = rotate_half(q, positions, rot["dims"], rot["base"], factor)
+            k = rotate_half(k, positions, rot["dims"], rot["base"], factor)
         return q, k, v
 
     def _attend(self, mem, q, k, v, positions, scale, H, sink=None, temp=None, talk=None):
@@ -217,6 +218,8 @@ class PlainSavidra:
             x = one_plus_norm(self.alpha * x + self._mixer(i, layer, h, positions, shared), w[f"l{i}.norm1"], self.eps)
             if layer.get("mlp") is not None:
                 x = one_plus_norm(self.alpha * x + self._ff(i, x), w[f"l{i}.norm2"], self.eps)
+            elif f"l{i}.norm2" in w:      # a second norm without a feed-forward: nothing is added
+                x = one_plus_norm(self.alpha * x, w[f"l{i}.norm2"], self.eps)
             if layers_out is not None:
                 layers_out.append(x.clone())
         x = one_plus_norm(x, w["final.norm"], self.eps)

@@ -22,7 +22,9 @@ import torch
 from plain_savidra import PlainSavidra
 
 # inner sizes of the delta branch's decay and gate products: a tensor's shape says them, the configuration does not
-RANKS = {"A": (3, 5), "B": (6, 2), "C": (16, 8), "D": (4, 4)}
+RANKS = {"A": (3, 5), "B": (6, 2), "C": (16, 8), "D": (4, 4), "E": (2, 3)}
+# layers without a feed-forward whose checkpoint nevertheless holds a second norm
+BARE_SECOND_NORM = {("E", 1)}
 
 
 def _rot(dims, base, factor=None):
@@ -99,8 +101,18 @@ SAVI_D = {
     ],
 }
 
-CONFIGS = {"A": SAVI_A, "B": SAVI_B, "C": SAVI_C, "D": SAVI_D}
-SEEDS = {"A": 3, "B": 13, "C": 23, "D": 43}
+# E: convolutions of one tap (nothing carried), a second norm in a layer without feed-forward, no key sizes named
+SAVI_E = {
+    "architecture": "Savidra", "vocab": 53, "width": 24, "norm": {"eps": 1e-6}, "postln_alpha": 0.5,
+    "layers": [
+        {"type": "parallel", "mixer": _side(_attn(2, 2, 6, 6, 0.4, _rot(6, 30.0), conv=1), _delta(2, 2, 4, 4, 1), 1.0, 0.9),
+         "mlp": _dense(16)},
+        {"type": "attention", "mixer": _attn(2, 1, 8, 8, 0.35, None), "mlp": None},
+    ],
+}
+
+CONFIGS = {"A": SAVI_A, "B": SAVI_B, "C": SAVI_C, "D": SAVI_D, "E": SAVI_E}
+SEEDS = {"A": 3, "B": 13, "C": 23, "D": 43, "E": 53}
 
 
 def _draw(name: str, shape, seed: int) -> torch.Tensor:
@@ -170,6 +182,8 @@ def shapes(which: str) -> dict:
                         q + "q.conv": (G * D, r["conv"]), q + "k.conv": (G * D, r["conv"]), q + "v.conv": (H * V, r["conv"]),
                         q + "b": (H, w), q + "A_log": (H,), q + "norm": (V,), q + "a1": (ra, w), q + "a2": (H * D, ra),
                         q + "dt_bias": (H * D,), q + "g1": (rg, w), q + "g2": (H * V, rg), q + "o": (w, H * V)})
+        if (which, i) in BARE_SECOND_NORM:
+            out[p + "norm2"] = (w,)
         if layer.get("mlp") is not None:
             ff = layer["mlp"]["ff"]
             out.update({p + "norm2": (w,), p + "mlp.gate": (ff, w), p + "mlp.up": (ff, w), p + "mlp.down": (w, ff)})

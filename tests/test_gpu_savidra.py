@@ -170,14 +170,15 @@ def _attend(ops, q, keys, values, positions, page, dtype, scale, temp=None, sink
     k_cache, v_cache, perm = _paged(keys, values, page, dtype, seed)
     out = torch.empty((T, H, values.shape[2]), dtype=dtype, device=DEV)
     dev = lambda t: f32(t) if t is not None else None  # noqa: E731
-    more = {"blocks": dict(parts=1), "parts": dict(parts=3), "tiles": dict(cu_seqlens_q=i32([0, T]), max_q_len=T)}[how]
+    more = {"blocks": dict(parts=1), "parts": dict(parts=3), "tiles": dict(cu_seqlens_q=i32([0, T]), max_q_len=T, parts=1),
+            "tile parts": dict(cu_seqlens_q=i32([0, T]), max_q_len=T, parts=3)}[how]
     ops.attention_together(q.to(dtype).to(DEV), k_cache, v_cache, out, i32([0] * T), i32(positions), i32([perm]), scale,
                            head_scale=dev(temp), sink=dev(sink), talk=dev(talk), max_context_len=keys.shape[0], **more)
     return out
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("how", ["blocks", "parts", "tiles"])
+@pytest.mark.parametrize("how", ["blocks", "parts", "tiles", "tile parts"])
 @pytest.mark.parametrize("H,G,D,DV,page,n,sink,talk,temp", [
     (4, 2, 10, 6, 4, 70, True, False, False), (6, 3, 6, 4, 16, 131, False, True, True), (2, 1, 12, 20, 8, 64, True, True, True),
     (4, 2, 128, 32, 16, 300, True, False, False), (4, 2, 48, 32, 16, 257, False, True, True), (1, 1, 14, 3, 16, 65, False, True, False),
@@ -190,7 +191,7 @@ def test_attention_against_plain(dtype, how, H, G, D, DV, page, n, sink, talk, t
     tk = torch.eye(H) + 0.3 * rnd((H, H), 5) if talk else None
     tp = 1 + 0.3 * rnd((H,), 6) if temp else None
     rows = sorted({0, 1, 2, page - 1, page, n // 2, 63, 64, 65, n - 2, n - 1} & set(range(n)))
-    if how == "tiles":       # more than a tile of rows, the last tile not full
+    if how.startswith("tile"):       # more than a tile of rows, the last tile not full
         rows = sorted(set(rows) | set(range(max(0, n - 40), n, 2)))
     at = torch.tensor(rows)
     w = ps.softmax_weights(q[rows].double(), keys.double(), at, torch.arange(n), 0.3,
@@ -202,8 +203,9 @@ def test_attention_against_plain(dtype, how, H, G, D, DV, page, n, sink, talk, t
     close(got, want, dtype, "attention")
 
 
+@pytest.mark.parametrize("parts", [1, 2, 7])
 @pytest.mark.parametrize("talk", [False, True])
-def test_tiles_of_several_requests(talk):
+def test_tiles_of_several_requests(talk, parts):
     """Portions of three requests and a single token in one launch, each behind a different number of cached tokens:
     every block finds its request and tile from its index alone."""
     ops = gpu_ops()
@@ -237,7 +239,7 @@ def test_tiles_of_several_requests(talk):
     out = torch.empty((sum(lens), H, DV), dtype=dtype, device=DEV)
     ops.attention_together(torch.cat(qs).to(DEV), k_cache.to(DEV), v_cache.to(DEV), out, i32(seq_of), i32(positions),
                            tables.to(DEV), 0.2, talk=f32(tk) if talk else None, max_context_len=150, cu_seqlens_q=i32(cu),
-                           max_q_len=max(lens))
+                           max_q_len=max(lens), parts=parts)
     close(out, torch.cat(wants), dtype, "tiles of several requests")
 
 
@@ -280,7 +282,8 @@ def test_heads_that_take_each_others_weights(dtype):
 
 # ------------------------------------------------------------------ the engine
 
-LENGTHS = {"A": [1, 7, 33, 150, 64, 300], "B": [2, 19, 45, 260, 128], "C": [3, 40, 17, 270, 96, 161], "D": [1, 9, 70, 200]}
+LENGTHS = {"A": [1, 7, 33, 150, 64, 300], "B": [2, 19, 45, 260, 128], "C": [3, 40, 17, 270, 96, 161], "D": [1, 9, 70, 200],
+           "E": [1, 2, 50, 130]}
 F32_TOL = dict(max=1e-4, mean=2e-5)
 BF16_TOL = dict(max=6e-2, mean=1.2e-2)
 
@@ -310,7 +313,7 @@ def _check(steps, results, requests, which, dtype, what):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E"])
 @pytest.mark.parametrize("cut", ["whole", "tail", "portions", "mixed"])
 def test_cuts_match_plain(which, cut, dtype):
     requests = _requests(which)

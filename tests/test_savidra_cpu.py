@@ -19,7 +19,7 @@ from atom_amd.config.model_config import SavidraConfig
 from atom_amd.engine.core import StepEntry, load_model
 from atom_amd.weights.loader import expected_tensors
 
-LENGTHS = {"A": [1, 7, 33, 70], "B": [2, 19, 45, 64], "C": [3, 52], "D": [1, 30, 66]}
+LENGTHS = {"A": [1, 7, 33, 70], "B": [2, 19, 45, 64], "C": [3, 52], "D": [1, 30, 66], "E": [1, 2, 40]}
 
 
 def _requests(which, seed=0):
@@ -167,7 +167,7 @@ def test_config_reads_every_size_and_round_trips():
     assert [b.mixer.inner.value_mix for b in later.blocks if hasattr(b.mixer.inner, "value_mix")] == ["source", "blend"]
 
 
-@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E"])
 def test_names_and_shapes_are_the_designs(which):
     model, _ = load_model(st.folder(which), dtype=torch.float32, device="cpu")
     names = {name: tuple(shape) for name, (shape, _) in expected_tensors(model).items()}
@@ -216,7 +216,20 @@ def test_config_refuses_what_does_not_fit(path, value):
 # ------------------------------------------------------------------ the engine's bookkeeping
 
 
-@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
+def test_a_second_norm_without_feed_forward_and_single_taps():
+    """A checkpoint that holds ``norm2`` for a layer without feed-forward gets ``x <- norm2(alpha x)`` there; without
+    the tensor the step is left out.  Convolutions of one tap carry nothing."""
+    model, _ = load_model(st.folder("E"), dtype=torch.float32, device="cpu")
+    assert model.blocks[1].ffn is None and model.blocks[1].ffn_norm is not None
+    assert "l1.norm2" in expected_tensors(model)
+    assert build_model(model_config_from_dict(st.SAVI_E)).blocks[1].ffn_norm is None
+    tokens = st.ids("E", 20, 1)
+    without = {k: v for k, v in st.tensors("E").items() if k != "l1.norm2"}
+    other = ps.PlainSavidra(st.CONFIGS["E"], without).forward(tokens)
+    assert float((other - st.oracle("E", tokens)).abs().max()) > 1e-3
+
+
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E"])
 @pytest.mark.parametrize("cut", ["whole", "tail", "portions", "mixed"])
 def test_cuts_match_plain(which, cut):
     requests = _requests(which)
