@@ -362,8 +362,15 @@ __global__ void together_sum_parts_kernel(const float* __restrict__ ws_o, T* __r
   if (idx >= total) return;
   const size_t t = idx / row;
   const size_t e = idx - t * row;
+  // the loads of four parts are asked for together; the shares are still added in the order of the parts
+  const float* src = ws_o + t * parts * row + e;
   float sum = 0.f;
-  for (int p = 0; p < parts; ++p) sum += ws_o[(t * parts + p) * row + e];
+  int p = 0;
+  for (; p + 4 <= parts; p += 4) {
+    const float a = src[(size_t)p * row], b = src[(size_t)(p + 1) * row], c = src[(size_t)(p + 2) * row], d = src[(size_t)(p + 3) * row];
+    sum = (((sum + a) + b) + c) + d;
+  }
+  for (; p < parts; ++p) sum += src[(size_t)p * row];
   out[idx] = from_f32<T>(sum);
 }
 

@@ -77,14 +77,17 @@ together_tile_kernel(TogetherTileArgs a) {
   const int group = a.H / a.G;
   const int ps = a.page_size;
 
+  // A wave whose share of the heads is not full works a stand-in head (the block's first, with a query of zeros) and
+  // stores nothing for it: the loops below then have no branch around their loads.
   tg_bf16x8 qf[HPW][D / 32];
   float top[HPW], den[HPW], hs[HPW];
   bool own[HPW];
+  int head[HPW];
 #pragma unroll
   for (int u = 0; u < HPW; ++u) {
     const int hh = wave + kTileWaves * u;
     own[u] = hh < HB;
-    const int h = h0 + (own[u] ? hh : 0);
+    const int h = head[u] = h0 + (own[u] ? hh : 0);
     const bf16_t* qr = a.q + ((size_t)(t0 + (row_ok ? n : 0)) * a.H + h) * D + 8 * g4;
 #pragma unroll
     for (int j = 0; j < D / 32; ++j) {
@@ -103,7 +106,7 @@ together_tile_kernel(TogetherTileArgs a) {
   // The 16 key rows from base as this lane's part of the A operand of the first product (head u's key/value head).
   struct KeyRows { tg_bf16x8 f[D / 32]; };
   auto load_keys = [&](int u, int base) -> KeyRows {
-    const int h = h0 + wave + kTileWaves * u;
+    const int h = head[u];
     int key = base + n;                       // the key row this lane brings
     if (key > pos_hi) key = pos_hi;           // beyond the tile's last key: any valid row, masked in the scores
     const int page = table[key / ps], off = key - key / ps * ps;
@@ -132,7 +135,7 @@ together_tile_kernel(TogetherTileArgs a) {
     int key0 = base + 4 * g4;
     if (key0 > pos_hi) key0 = pos_hi & ~3;      // unseen by every query: any valid place, the weights are zero
     const int page = table[key0 / ps], off = key0 - key0 / ps * ps;
-    const int kvh = (h0 + wave + kTileWaves * u) / group;
+    const int kvh = head[u] / group;
     const bf16_t* vr = a.v_cache + (((size_t)page * a.G + kvh) * DV + n) * (size_t)ps + off;
     ValueRows v;
 #pragma unroll
@@ -153,19 +156,16 @@ together_tile_kernel(TogetherTileArgs a) {
   if (PASS != 2) {
   // every (query, head)'s maximum and sum; the next chunk's key rows are asked for before this chunk's are used
 #pragma unroll
-  for (int u = 0; u < HPW; ++u)
-    if (own[u] && start < stop) ahead[u] = load_keys(u, start);
+  for (int u = 0; u < HPW; ++u) ahead[u] = load_keys(u, start);
   for (int base = start; base < stop; base += kTileRows) {
     KeyRows now[HPW];
 #pragma unroll
     for (int u = 0; u < HPW; ++u) {
-      if (!own[u]) continue;
       now[u] = ahead[u];
-      if (base + kTileRows < stop) ahead[u] = load_keys(u, base + kTileRows);
+      ahead[u] = load_keys(u, base + kTileRows);    // past the last chunk: the tile's last key again, not used
     }
 #pragma unroll
     for (int u = 0; u < HPW; ++u) {
-      if (!own[u]) continue;
       const tg_f32x4 s = scores(u, now[u], base);
       const float cm = rows_max(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
       const float m_new = fmaxf(top[u], cm);
@@ -202,10 +202,9 @@ together_tile_kernel(TogetherTileArgs a) {
   }
 #pragma unroll
   for (int u = 0; u < HPW; ++u) {
-    if (!own[u]) continue;
     float m = top[u], l = den[u];
     if (a.sink != nullptr && row_ok) {
-      const float sk = a.sink[h0 + wave + kTileWaves * u] * kLog2e;
+      const float sk = a.sink[head[u]] * kLog2e;
       const float m_new = fmaxf(m, sk);
       l = l * exp2f(m - m_new) + exp2f(sk - m_new);
       m = m_new;
@@ -221,24 +220,20 @@ together_tile_kernel(TogetherTileArgs a) {
 #pragma unroll
     for (int t = 0; t < NDV; ++t) acc[u][t] = tg_f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int u = 0; u < HPW; ++u)
-    if (own[u] && start < stop) ahead[u] = load_keys(u, start);
+  for (int u = 0; u < HPW; ++u) ahead[u] = load_keys(u, start);
   int turn = 0;
   for (int base = start; base < stop; base += kTileRows, turn ^= 1) {
     KeyRows now[HPW];
     ValueRows vals[HPW];
 #pragma unroll
     for (int u = 0; u < HPW; ++u) {
-      if (!own[u]) continue;
       now[u] = ahead[u];
       vals[u] = load_values(u, base);          // in flight while the scores are formed
-      if (base + kTileRows < stop) ahead[u] = load_keys(u, base + kTileRows);
+      ahead[u] = load_keys(u, base + kTileRows);
     }
     tg_f32x4 w[HPW];
 #pragma unroll
     for (int u = 0; u < HPW; ++u) {
-      w[u] = tg_f32x4{0.f, 0.f, 0.f, 0.f};
-      if (!own[u]) continue;
       const tg_f32x4 s = scores(u, now[u], base);
 #pragma unroll
       for (int i = 0; i < 4; ++i) w[u][i] = exp2f(s[i] - top[u]) * den[u];   // exp2(-inf) = 0 where unseen
@@ -248,8 +243,7 @@ together_tile_kernel(TogetherTileArgs a) {
       __syncthreads();
 #pragma unroll
       for (int u = 0; u < HPW; ++u) {
-        if (!own[u]) continue;
-        const float* row = a.talk + (size_t)(wave + kTileWaves * u) * a.H;
+        const float* row = a.talk + (size_t)head[u] * a.H;
         tg_f32x4 m = {0.f, 0.f, 0.f, 0.f};
         for (int g = 0; g < a.H; ++g) {
           const float c = row[g];
@@ -261,7 +255,6 @@ together_tile_kernel(TogetherTileArgs a) {
     }
 #pragma unroll
     for (int u = 0; u < HPW; ++u) {
-      if (!own[u]) continue;
       tg_bf16x4 pb;
 #pragma unroll
       for (int i = 0; i < 4; ++i) pb[i] = (__bf16)w[u][i];

@@ -1729,10 +1729,10 @@ class HipKernels:
             if block_tables.shape[0] != seqs:
                 raise KernelError("attention: one block table row per request is needed")
             if parts is None:
-                # enough blocks for four a CU, every part with at least four chunks of 16 keys
+                # up to eight blocks a CU (their waves hide each other's waits for memory), every part with at least four chunks of 16 keys
                 blocks = (tokens // 16 + seqs + 1) * (1 if talk is not None else G)
                 reach = block_tables.shape[1] * page_size if max_context_len is None else max_context_len
-                parts = max(1, min(8, 4 * self.num_cus // blocks, reach // 64))
+                parts = max(1, min(8, 8 * self.num_cus // blocks, reach // 64))
             ws_ml = ws_o = None
             if parts > 1:
                 ws_ml = self.workspace("together_ml", tokens * H * parts * 2)
@@ -1750,7 +1750,8 @@ class HipKernels:
             reach = block_tables.shape[1] * page_size if max_context_len is None else max_context_len
             if window:
                 reach = min(reach, window + 63)
-            parts = max(1, min(-(-2 * self.num_cus // max(sets, 1)), -(-reach // 64))) if sets < self.num_cus else 1
+            # two blocks a CU where the keys allow, every part with at least two chunks of 64 keys
+            parts = max(1, min(-(-2 * self.num_cus // max(sets, 1)), reach // 128)) if sets < self.num_cus else 1
         ws_ml = ws_o = None
         if parts > 1:
             ws_ml = self.workspace("together_ml", tokens * H * parts * 2)

@@ -343,14 +343,14 @@ def savidra_pair(size: str) -> tuple[dict, dict]:
     }[size]
     kv = max(1, heads // 4)
     attn = {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "v_mix": True,
-            "rot": {"base": 1000000.0, "dims": 64}}
-    left = {"heads": heads // 2, "kv_heads": max(1, kv // 2), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "conv": 3,
-            "rot": {"base": 500000.0, "dims": 128, "scaling": {"factor": 8.0}}}
+            "rot": {"base": 100000.0, "dims": 64}}
+    left = {"heads": heads // 2, "kv_heads": max(1, kv // 2), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "conv": 4,
+            "rot": {"base": 10000.0, "dims": 128, "scaling": {"factor": 4.0}}}
     right = {"heads": heads // 2, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "conv": 4, "decay_rank": 64,
              "gate_rank": 64}
-    side = {"left": left, "right": right, "left_scale": 0.6, "right_scale": 1.1}
+    side = {"left": left, "right": right, "left_scale": 0.75, "right_scale": 0.9}
     dense = {"kind": "dense", "ff": ff}
-    savi = {"architecture": "Savidra", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "postln_alpha": 2.0,
+    savi = {"architecture": "Savidra", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "postln_alpha": 1.5,
             "layers": [{"type": "parallel", "mixer": side, "mlp": dense},
                        {"type": "attention", "mixer": attn, "mlp": dense},
                        {"type": "parallel", "mixer": side, "mlp": dense},

@@ -50,13 +50,13 @@ def _batch(lens, slots):
 
 
 @pytest.mark.parametrize("out_dtype", DTYPES)
-@pytest.mark.parametrize("width,terms", [(40, 1), (192, 2), (1000, 2), (4096, 1), (52, 4)])
+@pytest.mark.parametrize("width,terms", [(40, 1), (176, 2), (1000, 2), (4096, 1), (52, 4)])
 def test_norm_of_a_sum_becomes_the_stream(out_dtype, width, terms):
     ops = gpu_ops()
     rows, alpha, eps = 7, 1.5, 1e-5
     stream = rnd((rows, width), 1)
     ys = [rnd((rows, width), 10 + k).to(torch.bfloat16 if k % 2 else torch.float32) for k in range(terms)]
-    scales = [0.6, 1.1, -0.4, 2.0][:terms]
+    scales = [0.7, 1.3, -0.4, 2.0][:terms]
     w = 0.2 * rnd((width,), 3)
     total = alpha * stream.double() + sum(s * y.double() for s, y in zip(scales, ys))
     want = ps.one_plus_norm(total, w.double(), eps)
@@ -73,7 +73,7 @@ def test_norm_of_a_sum_becomes_the_stream(out_dtype, width, terms):
 
 @pytest.mark.parametrize("x_dtype", DTYPES)
 @pytest.mark.parametrize("out_dtype", DTYPES)
-@pytest.mark.parametrize("width,off", [(50, 3), (192, 0), (2048, 8)])
+@pytest.mark.parametrize("width,off", [(50, 3), (208, 0), (2048, 8)])
 def test_blend_with_the_previous_token_across_steps(x_dtype, out_dtype, width, off):
     """Two steps over three requests in slots 2, 0 and 3 (one sits the second step out, a new one starts in a slot
     whose row was cleared): the row before a request's first token of a step is what the slot holds."""
@@ -101,7 +101,7 @@ def test_blend_with_the_previous_token_across_steps(x_dtype, out_dtype, width, o
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,G,D,DV,rot,page,normed,blend", [(4, 2, 10, 6, 6, 4, True, None), (2, 1, 12, 20, 12, 16, True, "blend"),
-                                                           (3, 3, 7, 7, 0, 8, False, "keep"), (4, 2, 128, 32, 64, 16, True, "blend"),
+                                                           (3, 3, 7, 7, 0, 8, False, "keep"), (6, 3, 128, 64, 32, 16, True, "blend"),
                                                            (1, 1, 14, 3, 2, 16, True, "keep")])
 def test_norm_rotation_blend_and_page_write(dtype, H, G, D, DV, rot, page, normed, blend):
     ops = gpu_ops()
@@ -181,7 +181,7 @@ def _attend(ops, q, keys, values, positions, page, dtype, scale, temp=None, sink
 @pytest.mark.parametrize("how", ["blocks", "parts", "tiles", "tile parts"])
 @pytest.mark.parametrize("H,G,D,DV,page,n,sink,talk,temp", [
     (4, 2, 10, 6, 4, 70, True, False, False), (6, 3, 6, 4, 16, 131, False, True, True), (2, 1, 12, 20, 8, 64, True, True, True),
-    (4, 2, 128, 32, 16, 300, True, False, False), (4, 2, 48, 32, 16, 257, False, True, True), (1, 1, 14, 3, 16, 65, False, True, False),
+    (8, 2, 128, 32, 16, 300, True, False, False), (6, 2, 48, 16, 16, 257, False, True, True), (1, 1, 14, 3, 16, 65, False, True, False),
     (16, 4, 64, 64, 16, 200, False, True, True), (3, 3, 7, 7, 4, 5, False, False, False), (8, 2, 128, 128, 16, 300, False, True, True),
     (8, 8, 64, 128, 8, 100, True, True, False), (12, 3, 64, 32, 4, 90, True, False, True), (32, 2, 128, 64, 16, 150, True, False, False)])
 def test_attention_against_plain(dtype, how, H, G, D, DV, page, n, sink, talk, temp):
