@@ -298,16 +298,21 @@ attention_together_part_kernel(const T* __restrict__ q, const T* __restrict__ k_
     }
     return;
   }
-  // the parts' maxima and sums, in the order of the parts
-  for (int hh = tid; hh < HB; hh += kTogetherThreads) {
+  // the parts' maxima and sums: a wave a head, a lane a part, so that the loads go out together
+  for (int hh = wave; hh < HB; hh += waves) {
     const float* ml = a.ws_ml + ((size_t)t * a.H + h0 + hh) * a.parts * 2;
-    float m = a.sink != nullptr ? a.sink[h0 + hh] : -INFINITY;
-    for (int p = 0; p < a.parts; ++p) m = fmaxf(m, ml[2 * p]);
-    float l = a.sink != nullptr ? expf(a.sink[h0 + hh] - m) : 0.f;
-    for (int p = 0; p < a.parts; ++p)
-      if (ml[2 * p] != -INFINITY) l += ml[2 * p + 1] * expf(ml[2 * p] - m);
-    top[hh] = m;
-    den[hh] = 1.f / l;
+    float m = -INFINITY;
+    for (int p = lane; p < a.parts; p += kWave) m = fmaxf(m, ml[2 * p]);
+    m = wave_max(m);
+    if (a.sink != nullptr) m = fmaxf(m, a.sink[h0 + hh]);
+    float l = 0.f;
+    for (int p = lane; p < a.parts; p += kWave) {
+      const float mp = ml[2 * p];
+      if (mp != -INFINITY) l += ml[2 * p + 1] * expf(mp - m);
+    }
+    l = wave_sum(l);
+    if (a.sink != nullptr) l += expf(a.sink[h0 + hh] - m);
+    if (lane == 0) top[hh] = m, den[hh] = 1.f / l;
   }
   __syncthreads();
   float acc[kTogetherAcc];

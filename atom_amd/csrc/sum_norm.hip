@@ -32,6 +32,7 @@ sum_norm_kernel(float* __restrict__ stream, float alpha, SumTerms terms, const f
   __shared__ float scratch[16];
   const size_t base = (size_t)blockIdx.x * width;
   float ss = 0.f;
+#pragma unroll 4
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     float v = alpha != 0.f ? alpha * stream[base + i] : 0.f;
     // the terms by constant index, so that the argument's arrays stay in scalar registers
@@ -43,6 +44,7 @@ sum_norm_kernel(float* __restrict__ stream, float alpha, SumTerms terms, const f
   }
   float inv = 1.f;
   if (weight != nullptr) inv = 1.f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+#pragma unroll 4
   for (int i = threadIdx.x; i < width; i += blockDim.x) {   // a thread reads back what it wrote itself
     const float v = weight != nullptr ? row[i] * inv * weight[i] : row[i];
     stream[base + i] = v;
@@ -83,6 +85,7 @@ shift_rows_kernel(const TI* __restrict__ x, const float* __restrict__ mu, TO* __
   const int last = padding ? t : cu_seqlens[seq + 1] - 1;
   float* kept = slot >= 0 ? state + (size_t)slot * slot_stride + state_off : nullptr;
   const TI* row = x + (size_t)t * width;
+#pragma unroll 4
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     const float cur = to_f32(row[i]);
     float prev;
@@ -157,6 +160,7 @@ qkv_rot_write_kernel(const float* __restrict__ qkv, int ld, T* __restrict__ q_ou
   __syncthreads();
   const int slot = slots != nullptr ? slots[t] : -1;
   const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+#pragma unroll 4
   for (int e = threadIdx.x; e < Q + K; e += blockDim.x) {
     const bool is_k = e >= Q;
     const int j = is_k ? e - Q : e;
@@ -180,6 +184,7 @@ qkv_rot_write_kernel(const float* __restrict__ qkv, int ld, T* __restrict__ q_ou
     }
   }
   const float lam = (v_source != nullptr && v_blend != nullptr) ? v_blend[0] : 0.f;
+#pragma unroll 4
   for (int j = threadIdx.x; j < V; j += blockDim.x) {
     float v = vr[j];
     if (v_keep != nullptr) v_keep[(size_t)t * V + j] = v;
