@@ -31,6 +31,8 @@ struct TogetherArgs {
   int parts;          // > 1: the keys of a token are cut over this many blocks
   float* ws_ml;       // [tokens, H, parts, 2]: a part's maximum and sum
   float* ws_o;        // [tokens, parts, H, DV]: a part's share of the weighted sum
+  float* ws_s;        // [tokens, H, s_stride] or null: the scores of the first launch, kept for the second
+  long s_stride;      // at least the longest context
 };
 
 // The chunks [c0, c1) of a token's visible keys that part `part` takes, counted from the chunk that holds `first`.
@@ -279,6 +281,12 @@ attention_together_part_kernel(const T* __restrict__ q, const T* __restrict__ k_
       const int lo = base > first ? base : first;
       const int hi = base + kTogetherChunk - 1 < pos ? base + kTogetherChunk - 1 : pos;
       together_scores(a, k_cache, table, qs, s, h0, HB, base, lo, hi);
+      if (a.ws_s != nullptr) {   // a thread keeps the scores it formed itself
+        for (int item = tid; item < HB * kTogetherChunk; item += kTogetherThreads) {
+          const int hh = item / kTogetherChunk, key = base + item - hh * kTogetherChunk;
+          if (key >= lo && key <= hi) a.ws_s[((size_t)t * a.H + h0 + hh) * a.s_stride + key] = s[item];
+        }
+      }
       __syncthreads();
       for (int hh = wave; hh < HB; hh += waves) {
         const float v = s[hh * kTogetherChunk + lane];
@@ -322,7 +330,14 @@ attention_together_part_kernel(const T* __restrict__ q, const T* __restrict__ k_
   for (int base = base0; base < base1; base += kTogetherChunk) {
     const int lo = base > first ? base : first;
     const int hi = base + kTogetherChunk - 1 < pos ? base + kTogetherChunk - 1 : pos;
-    together_scores(a, k_cache, table, qs, s, h0, HB, base, lo, hi);
+    if (a.ws_s != nullptr) {
+      for (int item = tid; item < HB * kTogetherChunk; item += kTogetherThreads) {
+        const int hh = item / kTogetherChunk, key = base + item - hh * kTogetherChunk;
+        s[item] = (key >= lo && key <= hi) ? a.ws_s[((size_t)t * a.H + h0 + hh) * a.s_stride + key] : -INFINITY;
+      }
+    } else {
+      together_scores(a, k_cache, table, qs, s, h0, HB, base, lo, hi);
+    }
     for (int r = tid; r <= hi / a.page_size - base / a.page_size; r += kTogetherThreads) pg[r] = table[base / a.page_size + r];
     for (int item = tid; item < HB * kTogetherChunk; item += kTogetherThreads) {
       const int hh = item / kTogetherChunk;
@@ -400,7 +415,8 @@ ATOM_EXPORT int atom_attention_together(const void* q, const void* k_cache, cons
                                         const int* token_seq, const int* positions, const int* block_tables,
                                         int max_blocks, int tokens, int H, int G, int D, int DV, int page_size,
                                         float scale, const float* head_scale, const float* sink, const float* talk,
-                                        int window, int parts, float* ws_ml, float* ws_o, hipStream_t stream) {
+                                        int window, int parts, float* ws_ml, float* ws_o, float* ws_s, long s_stride,
+                                        hipStream_t stream) {
   if (tokens < 0 || H <= 0 || G <= 0 || D <= 0 || DV <= 0 || page_size <= 0 || max_blocks <= 0) return ATOM_BAD_SHAPE;
   if (H % G || window < 0) return ATOM_BAD_SHAPE;
   if (q == nullptr || k_cache == nullptr || v_cache == nullptr || out == nullptr) return ATOM_BAD_SHAPE;
@@ -413,7 +429,8 @@ ATOM_EXPORT int atom_attention_together(const void* q, const void* k_cache, cons
   if (tokens == 0) return ATOM_OK;
   if (parts < 1 || parts > 65535 || (parts > 1 && (ws_ml == nullptr || ws_o == nullptr))) return ATOM_BAD_SHAPE;
   TogetherArgs a{token_seq, positions, block_tables, max_blocks, H, G, D, DV, page_size, window, scale, head_scale, sink,
-                 talk, parts, ws_ml, ws_o};
+                 talk, parts, ws_ml, ws_o, parts > 1 ? ws_s : nullptr, s_stride};
+  if (a.ws_s != nullptr && s_stride < (long)max_blocks * page_size) return ATOM_BAD_SHAPE;
   dim3 grid(tokens, mixes ? 1 : G, parts), block(kTogetherThreads);
   if (parts == 1) {
     ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((attention_together_kernel<T>), grid, block, smem, stream, (const T*)q,

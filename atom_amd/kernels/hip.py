@@ -1752,15 +1752,19 @@ class HipKernels:
                 reach = min(reach, window + 63)
             # two blocks a CU where the keys allow, every part with at least two chunks of 64 keys
             parts = max(1, min(-(-2 * self.num_cus // max(sets, 1)), reach // 128)) if sets < self.num_cus else 1
-        ws_ml = ws_o = None
+        ws_ml = ws_o = ws_s = None
+        stride = block_tables.shape[1] * page_size
         if parts > 1:
             ws_ml = self.workspace("together_ml", tokens * H * parts * 2)
             ws_o = self.workspace("together_o", tokens * parts * H * DV)
+            if tokens * H * stride <= 1 << 24:
+                # the second launch reads the first one's scores instead of the keys again (up to 64 MB of them)
+                ws_s = self.workspace("together_s", tokens * H * stride)
         self._done("attention_together", self.lib.atom_attention_together(
             _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), self._code(q), _ptr(token_seq), _ptr(positions),
             _ptr(block_tables), block_tables.shape[1], tokens, H, G, D, DV, page_size, ctypes.c_float(scale),
-            _ptr(head_scale), _ptr(sink), _ptr(talk), int(window or 0), int(parts), _ptr(ws_ml), _ptr(ws_o),
-            self._stream()))
+            _ptr(head_scale), _ptr(sink), _ptr(talk), int(window or 0), int(parts), _ptr(ws_ml), _ptr(ws_o), _ptr(ws_s),
+            ctypes.c_long(stride), self._stream()))
         return out
 
     def router_choose(self, logits, correction, top: int, renormalize: bool = False):
