@@ -56,7 +56,13 @@ struct AttnParams {
   const int* slots;       // [tokens] cache slot of each token's key and value (-1: none)
   float eps;
   int write_kv;           // 0: the keys and values are another layer's, already written
+  // A learned number per query head that joins the softmax's denominator as exp(sink[h]), unscaled, with no key and
+  // no value (null: none).  It is where a row's running maximum and sum start: as if a key with that score and a
+  // value of zeros had been seen already; of the parts of a row's keys only the first starts so.
+  const float* sink;      // [Hq]
 };
+
+constexpr float kSinkLog2e = 1.4426950408889634f;
 
 __device__ __forceinline__ s16x4 as_s16x4(bf16x4 v) { return __builtin_bit_cast(s16x4, v); }
 
@@ -195,6 +201,14 @@ __global__ void __launch_bounds__(kWave) attention_mfma_kernel(AttnParams p) {
     run_sum[rt] = 0.f;
 #pragma unroll
     for (int t = 0; t < DT; ++t) acc[rt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  if (p.sink != nullptr && (!DECODE || part == 0)) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      if (!row_ok[rt]) continue;
+      run_max[rt] = p.sink[DECODE ? head0 + rt * 16 + r16 : head0] * kSinkLog2e;
+      run_sum[rt] = g == 0 ? 1.f : 0.f;    // the sum is kept in four lanes a row and added up at the end
+    }
   }
 
   // One block of 16 keys in registers: the K rows as the first product's A operand, the V^T rows
@@ -419,6 +433,14 @@ __global__ void __launch_bounds__(TOGETHER ? 8 * kWave : kWave, (D <= 128 ? 2 : 
     run_sum[rt] = 0.f;
 #pragma unroll
     for (int t = 0; t < DT; ++t) acc[rt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  if (p.sink != nullptr && part == 0) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      if (rt * 16 + r16 >= group) continue;
+      run_max[rt] = p.sink[head0 + rt * 16 + r16] * kSinkLog2e;
+      run_sum[rt] = g == 0 ? 1.f : 0.f;
+    }
   }
 
   struct Step {
@@ -939,6 +961,14 @@ __global__ void __launch_bounds__(256 * KS, (D <= 128 && KS == 1 ? 2 : 1)) atten
 #pragma unroll
     for (int t = 0; t < DT; ++t) acc[rt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
+  if (p.sink != nullptr && part == 0) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      if (!row_ok[rt]) continue;
+      run_max[rt] = p.sink[head] * kSinkLog2e;
+      run_sum[rt] = g == 0 ? 1.f : 0.f;
+    }
+  }
 
   // ---- moving a tile: piece q of K is (key q / (D/8), 8 elements at (q % (D/8)) * 8);
   //      piece q of V^T is (d = q / (TK/8), the 8 keys at (q % (TK/8)) * 8)
@@ -1267,7 +1297,7 @@ ATOM_EXPORT int atom_attention_decode(const void* q, const void* k_cache, const 
                                       const int* cu_q, const int* ctx_lens, const int* block_tables, int max_blocks,
                                       int seq_offset, int seqs, int hq, int hkv, int d, int page_size, float scale,
                                       int window, int chunk, float softcap, int parts, float* ws_o, float* ws_ml,
-                                      hipStream_t stream) {
+                                      const float* sink, hipStream_t stream) {
   if (int st = check_common(hq, hkv, d, page_size, max_blocks)) return st;
   if (seqs < 0 || parts < 1 || seq_offset < 0 || window < 0 || chunk < 0 || softcap < 0.f) return ATOM_BAD_SHAPE;
   if (softcap > 0.f && !(scale > 0.f)) return ATOM_UNSUPPORTED;
@@ -1281,6 +1311,7 @@ ATOM_EXPORT int atom_attention_decode(const void* q, const void* k_cache, const 
   p.ws_o = ws_o; p.ws_ml = ws_ml; p.max_blocks = max_blocks; p.hq = hq; p.hkv = hkv; p.page_size = page_size;
   p.window = window; p.seq_offset = seq_offset; p.parts = parts; p.scale_log2 = scale * 1.4426950408889634f;
   p.chunk = chunk;
+  p.sink = sink;
   if (softcap > 0.f) { p.cap_in = scale / softcap; p.cap_out = softcap / scale; }
   p.page_shift = page_shift_of(page_size);
 #define CALL(DD) return launch_decode<DD, false>(p, seqs, stream)
@@ -1339,7 +1370,7 @@ ATOM_EXPORT int atom_attention_prefill(const void* q, const void* k_cache, const
                                        const int* cu_q, const int* ctx_lens, const int* block_tables, int max_blocks,
                                        const int* tiles, int num_tiles, int rows_per_tile, int tiled, int hq, int hkv,
                                        int d, int page_size, float scale, int window, int chunk, float softcap,
-                                       hipStream_t stream) {
+                                       const float* sink, hipStream_t stream) {
   if (int st = check_common(hq, hkv, d, page_size, max_blocks)) return st;
   if (num_tiles < 0 || !tiles || window < 0 || chunk < 0 || softcap < 0.f) return ATOM_BAD_SHAPE;
   if (softcap > 0.f && !(scale > 0.f)) return ATOM_UNSUPPORTED;
@@ -1350,6 +1381,7 @@ ATOM_EXPORT int atom_attention_prefill(const void* q, const void* k_cache, const
   p.ws_o = nullptr; p.ws_ml = nullptr; p.max_blocks = max_blocks; p.hq = hq; p.hkv = hkv; p.page_size = page_size;
   p.window = window; p.seq_offset = 0; p.parts = 1; p.scale_log2 = scale * 1.4426950408889634f;
   p.chunk = chunk;
+  p.sink = sink;
   if (softcap > 0.f) { p.cap_in = scale / softcap; p.cap_out = softcap / scale; }
   p.page_shift = page_shift_of(page_size);
   p.num_tiles = num_tiles;

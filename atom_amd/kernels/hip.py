@@ -576,7 +576,8 @@ class HipKernels:
             *self._sum_args(qkv), self._stream()))
         return q_out
 
-    def _attention_mfma(self, q, k_cache, v_cache, out, meta, scale, window, parts=None, softcap=None, chunk=None):
+    def _attention_mfma(self, q, k_cache, v_cache, out, meta, scale, window, parts=None, softcap=None, chunk=None,
+                        sink=None):
         tokens, hq, d = q.shape
         _, hkv, page_size, _ = k_cache.shape
         self._check("cu_seqlens_q", meta.cu_seqlens_q, torch.int32, (meta.num_seqs + 1,))
@@ -601,7 +602,7 @@ class HipKernels:
             self._done("attention_prefill", self.lib.atom_attention_prefill(
                 _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(meta.cu_seqlens_q), _ptr(meta.context_lens),
                 _ptr(bt), bt.shape[1], _ptr(tiles), tiles.shape[0], rows, tiled, hq, hkv, d, page_size,
-                ctypes.c_float(scale), int(window or 0), int(chunk or 0), ctypes.c_float(softcap or 0.0),
+                ctypes.c_float(scale), int(window or 0), int(chunk or 0), ctypes.c_float(softcap or 0.0), _ptr(sink),
                 self._stream()))
         seqs = meta.num_seqs - meta.num_prefill
         if seqs:
@@ -618,7 +619,7 @@ class HipKernels:
                 _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(meta.cu_seqlens_q), _ptr(meta.context_lens),
                 _ptr(bt), bt.shape[1], meta.num_prefill, seqs, hq, hkv, d, page_size, ctypes.c_float(scale),
                 int(window or 0), int(chunk or 0), ctypes.c_float(softcap or 0.0), parts, _ptr(ws_o), _ptr(ws_ml),
-                self._stream()))
+                _ptr(sink), self._stream()))
         return out
 
     def _prefill_in_halves(self, blocks: int, meta) -> bool:
@@ -699,10 +700,12 @@ class HipKernels:
 
     def paged_attention(self, q, k_cache, v_cache, out, meta: AttentionMeta, scale: float,
                         window: int | None = None, parts: int | None = None, softcap: float | None = None,
-                        chunk: int | None = None):
+                        chunk: int | None = None, sink=None):
         """Attention of the step's queries over the pages.  ``window``: only the latest that many keys;
         ``chunk``: only the keys of the query's own run of that many positions, counted from position 0;
-        ``softcap``: a score s becomes ``softcap * tanh(s / softcap)``."""
+        ``softcap``: a score s becomes ``softcap * tanh(s / softcap)``; ``sink`` (float32 [Hq]): ``exp(sink[h])``
+        joins head h's denominator with no key and no value (the matrix-core kernels only: ask
+        ``takes_sink`` first)."""
         tokens, hq, d = q.shape
         _, hkv, page_size, _ = k_cache.shape
         dt = q.dtype
@@ -722,14 +725,24 @@ class HipKernels:
         group = hq // hkv
         if softcap and not scale > 0:
             raise KernelError("attention: a cap on the scores needs a positive scale")
+        if sink is not None:
+            self._check("sink", sink, torch.float32, (hq,))
         if (dt == torch.bfloat16 and self.use_mfma_attention
                 and self.lib.atom_attention_mfma_supports(d, page_size, group)):
-            return self._attention_mfma(q, k_cache, v_cache, out, meta, scale, window, parts, softcap, chunk)
+            return self._attention_mfma(q, k_cache, v_cache, out, meta, scale, window, parts, softcap, chunk, sink)
+        if sink is not None:
+            raise KernelError("attention: the general kernel has no sink; ask takes_sink before")
         self._done("paged_attention", self.lib.atom_paged_attention_generic(
             _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(meta.token_seq), _ptr(meta.positions),
             _ptr(meta.block_tables), meta.block_tables.shape[1], self._code(q), tokens, hq, hkv, d, page_size,
             ctypes.c_float(scale), int(window or 0), int(chunk or 0), ctypes.c_float(softcap or 0.0), self._stream()))
         return out
+
+    def takes_sink(self, dtype, head_dim: int, value_dim: int, page_size: int, group: int) -> bool:
+        """Whether ``paged_attention`` takes a ``sink`` for these sizes: the matrix-core kernels, whose keys and
+        values have one head size."""
+        return bool(dtype == torch.bfloat16 and self.use_mfma_attention and head_dim == value_dim
+                    and self.lib.atom_attention_mfma_supports(head_dim, page_size, group))
 
     def _library_slices(self, m: int, n: int, k: int) -> int:
         """Into how many slices of K a product that goes to the BLAS library is cut when its reader can add

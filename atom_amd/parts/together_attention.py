@@ -19,18 +19,27 @@
 
 ``score = (q . k) * scale``.  Keys live in pages [pages, G, page, dim], values in pages [pages, G, vdim, page].  The
 projection's sums stay float32 through convolution, norm and rotation; q and the pages take the step's type.
+
+Without head mixing and temperature, and with values of the keys' size, nothing needs the heads together: the step
+then runs the paged attention kernels of ``GroupedQueryAttention`` (one walk over the keys; the sink is where a row's
+running maximum and sum start) where they take the sizes, and this mixer prepares their tiles of query rows.
 """
 
 from __future__ import annotations
 
 import torch
 
+from .attention import GroupedQueryAttention
 from .base import MIXERS, POSITION_ENCODINGS, KVCacheNeed, Mixer, ParamSpec, PartChoice, StateNeed
 from .parallel import JointNeed
 
 
-class TogetherAttention(Mixer):
+class TogetherAttention(GroupedQueryAttention):
+    """Shares with ``GroupedQueryAttention`` only what the paged kernels want to know about a step (``step_key``,
+    ``prepare_step``, the batch record); parameters, memory and the forward pass are its own."""
+
     graph_safe = True
+    accepts_deferred = False
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, scale: float,
                  value_dim: int | None = None, norm_eps: float = 1e-6, qkv_bias: bool = False, out_bias: bool = False,
@@ -38,7 +47,7 @@ class TogetherAttention(Mixer):
                  head_temperature: bool = False, sink: bool = False, talk: bool = False,
                  value_mix: str | None = None, window: int | None = None, prefix: str = "",
                  names: dict[str, str] | None = None):
-        super().__init__(prefix)
+        Mixer.__init__(self, prefix)
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} key/value heads")
         if value_mix not in (None, "source", "blend"):
@@ -57,6 +66,17 @@ class TogetherAttention(Mixer):
 
     def children(self):
         return [self.rope] if self.rope is not None else []
+
+    @property
+    def one_walk(self) -> bool:
+        """Whether nothing in this mixer needs a token's heads together."""
+        return not self.talk and not self.head_temperature and self.value_dim == self.head_dim
+
+    def step_key(self):
+        return super().step_key() if self.one_walk else None
+
+    def prepare_step(self, batch):
+        return super().prepare_step(batch) if self.one_walk else {}
 
     @property
     def channels(self) -> int:
@@ -125,6 +145,11 @@ class TogetherAttention(Mixer):
                           ctx.slot_mappings[group], H, G, D, DV, ctx.page_sizes[group], self.norm_eps,
                           v_source=source, v_blend=self.p("vmix") if source is not None else None, v_keep=keep)
         out = torch.empty((T, H, DV), dtype=ctx.dtype, device=x.device)
+        takes = getattr(ops, "takes_sink", None)
+        if self.one_walk and takes is not None and takes(ctx.dtype, D, DV, ctx.page_sizes[group], H // G):
+            ops.paged_attention(q, pages.k_cache, pages.v_cache, out, self._meta(ctx, group), self.scale, self.window,
+                                sink=self.p("sink"))
+            return ops.linear(out.view(T, H * DV), self.params["o.weight"], self.p("o.bias"), out_dtype=torch.float32)
         ops.attention_together(q, pages.k_cache, pages.v_cache, out, ctx.token_seq, ctx.positions,
                                ctx.block_tables[group], self.scale, head_scale=self.p("temp"), sink=self.p("sink"),
                                talk=self.p("talk"), window=self.window, max_context_len=ctx.max_context_len,

@@ -80,14 +80,14 @@ SAVI_B = {
     ],
 }
 
-# C: sizes that matrix-core kernels take
+# C: sizes that matrix-core kernels take; one attention layer whose values have the keys' size, one whose have not
 SAVI_C = {
     "architecture": "Savidra", "vocab": 160, "width": 64, "norm": {"eps": 1e-5}, "postln_alpha": 2.5,
     "layers": [
         {"type": "parallel", "mixer": _side(_attn(4, 2, 64, 64, 0.17, _rot(32, 10000.0, 6.0), conv=4),
                                             _delta(2, 1, 32, 64, 4), 0.8, 0.9), "mlp": _dense(96)},
-        {"type": "attention", "mixer": _attn(4, 2, 64, 32, 0.11, _rot(32, 50000.0), v_mix=True), "mlp": _dense(64)},
-        {"type": "attention", "mixer": _attn(2, 2, 128, 32, 0.09, _rot(64, 1000.0), v_mix=True), "mlp": _dense(80)},
+        {"type": "attention", "mixer": _attn(4, 2, 64, 64, 0.11, _rot(32, 50000.0), v_mix=True), "mlp": _dense(64)},
+        {"type": "attention", "mixer": _attn(2, 2, 128, 64, 0.09, _rot(64, 1000.0), v_mix=True), "mlp": _dense(80)},
     ],
 }
 

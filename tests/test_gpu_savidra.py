@@ -280,6 +280,46 @@ def test_heads_that_take_each_others_weights(dtype):
     close(got[0, 1], values[3, 1].to(dtype), dtype, "head 1")
 
 
+# ------------------------------------------------------------------ a sink in the one-walk kernels
+
+
+@pytest.mark.parametrize("H,G,D,page", [(4, 2, 64, 16), (8, 2, 128, 16), (2, 2, 64, 8), (16, 1, 128, 16), (6, 6, 32, 4)])
+@pytest.mark.parametrize("cached,fresh", [(0, 70), (37, 200), (300, 33), (700, 1), (5, 1), (64, 2)])
+def test_sink_in_the_paged_kernels(H, G, D, page, cached, fresh):
+    """A prompt portion behind cached tokens, or a single token whose keys are cut over several parts: the sink is
+    where a row's running maximum and sum start, and counts once."""
+    from atom_amd.kernels.hip import AttentionMeta
+
+    ops = gpu_ops()
+    dtype, n = torch.bfloat16, cached + fresh
+    if not ops.takes_sink(dtype, D, D, page, H // G):
+        pytest.skip("the matrix-core kernels do not take these sizes")
+    q, keys, values = rnd((n, H, D), 1).to(dtype), rnd((n, G, D), 2).to(dtype), rnd((n, G, D), 3).to(dtype)
+    sink = 2.0 * rnd((H,), 4) + 1.0
+    k_cache, v_cache, perm = _paged(keys, values, page, dtype, n)
+    rows = list(range(cached, n))
+    at = torch.tensor(rows)
+    w = ps.softmax_weights(q[rows].double(), keys.double(), at, torch.arange(n), 0.25, sink=sink.double())
+    want = ps.apply_weights(w, values.double(), H).view(fresh, H, D)
+    for parts in ([None] if fresh > 1 else [None, 1, 3, 8]):
+        meta = AttentionMeta(token_seq=i32([0] * fresh), positions=i32(rows), block_tables=i32([perm]),
+                             cu_seqlens_q=i32([0, fresh]), context_lens=i32([n]), num_seqs=1, num_tokens=fresh,
+                             max_q_len=fresh, max_context_len=n, page_size=page, num_prefill=1 if fresh > 1 else 0)
+        if fresh > 1:
+            short, tall = ops.attention_tile_rows(dtype, D, page, H // G, fresh)
+            if short:
+                meta.rows_per_tile = short
+                meta.prefill_tiles = i32([[0, r] for r in range(0, fresh, short)])
+            if tall:
+                meta.tiles_by_rows = {tall: i32([[0, r] for r in range(0, fresh, tall)])}
+        out = torch.empty((fresh, H, D), dtype=dtype, device=DEV)
+        ops.paged_attention(q[rows].to(DEV).contiguous(), k_cache, v_cache, out, meta, 0.25, parts=parts, sink=f32(sink))
+        close(out, want, dtype, f"parts {parts}")
+        plain = torch.empty_like(out)
+        ops.paged_attention(q[rows].to(DEV).contiguous(), k_cache, v_cache, plain, meta, 0.25, parts=parts)
+        assert float((plain.float() - out.float()).abs().max()) > 1e-3, "the sink changes nothing"
+
+
 # ------------------------------------------------------------------ the engine
 
 LENGTHS = {"A": [1, 7, 33, 150, 64, 300], "B": [2, 19, 45, 260, 128], "C": [3, 40, 17, 270, 96, 161], "D": [1, 9, 70, 200],
