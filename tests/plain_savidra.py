@@ -57,14 +57,18 @@ def rotate_half(x, positions, dims, base, factor=1.0):
     return torch.cat([u * c - v * s, v * c + u * s, x[..., dims:]], -1)
 
 
-def softmax_weights(q, k, positions_q, positions_k, scale, sink=None, temp=None):
-    """q [Tq, H, D], k [Tk, G, D] -> weights [H, Tq, Tk], causal by position, an optional sink in the denominator."""
+def softmax_weights(q, k, positions_q, positions_k, scale, sink=None, temp=None, window=None):
+    """q [Tq, H, D], k [Tk, G, D] -> weights [H, Tq, Tk], causal by position, an optional sink in the denominator;
+    ``window``: a query sees itself and the ``window - 1`` positions before it (the design has none; the engine's
+    kernels offer it)."""
     H, G = q.shape[1], k.shape[1]
     kk = k.repeat_interleave(H // G, dim=1)
     s = torch.einsum("ihd,jhd->hij", q, kk) * scale
     if temp is not None:
         s = s * temp[:, None, None]
     seen = positions_k[None, :] <= positions_q[:, None]
+    if window:
+        seen = seen & (positions_k[None, :] > positions_q[:, None] - window)
     s = s.masked_fill(~seen[None], -math.inf)
     m = s.max(-1, keepdim=True).values
     if sink is not None:

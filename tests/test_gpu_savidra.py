@@ -163,7 +163,8 @@ def _paged(keys, values, page, dtype, order_seed):
     return k_cache.to(DEV), v_cache.to(DEV), perm
 
 
-def _attend(ops, q, keys, values, positions, page, dtype, scale, temp=None, sink=None, talk=None, seed=0, how="blocks"):
+def _attend(ops, q, keys, values, positions, page, dtype, scale, temp=None, sink=None, talk=None, seed=0, how="blocks",
+            window=None):
     """``how``: "blocks" (a block a token and set of heads), "parts" (a token's keys cut over three blocks), "tiles"
     (the rows as a prompt portion of one request: the matrix cores where the sizes allow)."""
     T, H, D = q.shape
@@ -173,7 +174,8 @@ def _attend(ops, q, keys, values, positions, page, dtype, scale, temp=None, sink
     more = {"blocks": dict(parts=1), "parts": dict(parts=3), "tiles": dict(cu_seqlens_q=i32([0, T]), max_q_len=T, parts=1),
             "tile parts": dict(cu_seqlens_q=i32([0, T]), max_q_len=T, parts=3)}[how]
     ops.attention_together(q.to(dtype).to(DEV), k_cache, v_cache, out, i32([0] * T), i32(positions), i32([perm]), scale,
-                           head_scale=dev(temp), sink=dev(sink), talk=dev(talk), max_context_len=keys.shape[0], **more)
+                           head_scale=dev(temp), sink=dev(sink), talk=dev(talk), max_context_len=keys.shape[0],
+                           window=window, **more)
     return out
 
 
@@ -262,6 +264,35 @@ def test_a_far_key_is_found_and_a_later_one_is_not(dtype, far):
     # a sink as large as the key's score takes half of the weight and brings no value
     got = _attend(ops, q, keys, values, [n - 1], page, dtype, 1.0, sink=torch.tensor([36.0, -40.0]))
     assert 20.0 < float(got[0, 0].float().mean()) < 30.0 and float(got[0, 1].float().min()) > 45.0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("how", ["blocks", "parts", "tiles", "tile parts"])
+@pytest.mark.parametrize("window", [1, 9, 16, 64, 65, 200])
+def test_a_window_holds_the_token_itself_and_the_ones_before(dtype, how, window):
+    """The design has no window; the kernels offer one to others.  A key made to stand out is seen by the query
+    ``window - 1`` positions after it and not by the next, with and without mixed heads, and everything matches the
+    plain weights."""
+    ops = gpu_ops()
+    n, H, G, D, DV, page = 300, 4, 2, 64, 32, 16
+    q, keys, values = 0.3 * rnd((n, H, D), 1), 0.3 * rnd((n, G, D), 2), rnd((n, G, DV), 3)
+    at_key = 120
+    q[:, :, 0], keys[at_key, :, 0] = 5.0, 8.0
+    values[at_key] = 40.0
+    q, keys, values = q.to(dtype), keys.to(dtype), values.to(dtype)
+    tk = torch.eye(H) + 0.2 * rnd((H, H), 5)
+    rows = sorted({at_key, at_key + window - 1, at_key + window, 0, 63, 64, n - 1} & set(range(n)))
+    at = torch.tensor(rows)
+    for talk in (None, tk):
+        w = ps.softmax_weights(q[rows].double(), keys.double(), at, torch.arange(n), 0.5, window=window)
+        if talk is not None:
+            w = torch.einsum("hg,gij->hij", talk.double(), w)
+        want = ps.apply_weights(w, values.double(), H).view(len(rows), H, DV)
+        got = _attend(ops, q[rows], keys, values, rows, page, dtype, 0.5, talk=talk, seed=window, how=how, window=window)
+        close(got, want, dtype, f"window {window}")
+        if talk is None and at_key + window < n:
+            inside, outside = rows.index(at_key + window - 1), rows.index(at_key + window)
+            assert float(got[inside].float().mean()) > 30.0 and float(got[outside].float().abs().mean()) < 10.0
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
